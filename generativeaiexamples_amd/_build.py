@@ -112,7 +112,9 @@ def build_c(jobs: int = 8, force: bool = False, verbose: bool = False) -> Path:
     inc, torch_lib, abi = _torch_paths()
     pyinc = sysconfig.get_paths()["include"]
     hip_flags = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", f"-I{CSRC / 'include'}",
-                 "-munsafe-fp-atomics", "-Wno-unused-result"]
+                 "-munsafe-fp-atomics", "-Wno-unused-result",
+                 # scalar fp32 code generation only: the compiler forms no packed-fp32 (v_pk_*_f32) instructions
+                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     cxx_flags = ["-O2", "-std=c++17", "-fPIC", f"-I{CSRC / 'include'}", f"-I{pyinc}",
                  "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", f"-D_GLIBCXX_USE_CXX11_ABI={abi}",
                  "-DTORCH_EXTENSION_NAME=_C", "-DTORCH_API_INCLUDE_EXTENSION_H", "-Wno-deprecated-declarations",
