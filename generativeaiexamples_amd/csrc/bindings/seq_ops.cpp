@@ -1,0 +1,238 @@
+// PyTorch bindings of the sequence-mixer kernels with a 32-bit residual / state (norm_f32.hip, attention_window.hip,
+// recurrent.hip). Shape / dtype checks on the host, a launch on the current stream, no allocation: graph-capturable.
+// Activation tensors are bf16 or fp32 (all of one call alike); per-channel tables and states are fp32.
+#include <torch/extension.h>
+#include <c10/hip/HIPStream.h>
+
+#include "gai_kernels.h"
+
+namespace {
+
+using at::Tensor;
+using c10::optional;
+
+hipStream_t cur_stream() { return c10::hip::getCurrentHIPStream().stream(); }
+
+int act_dt(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda(), name, " must be a GPU tensor");
+  TORCH_CHECK(t.scalar_type() == at::kFloat || t.scalar_type() == at::kBFloat16, name, " must be bf16 or fp32");
+  return t.scalar_type() == at::kFloat ? 1 : 0;
+}
+void same_dt(const Tensor& t, int dt, const char* name) { TORCH_CHECK(act_dt(t, name) == dt, name, ": dtype differs"); }
+const float* f32(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous(), name, " must be a contiguous fp32 GPU tensor");
+  return t.data_ptr<float>();
+}
+float* f32w(Tensor& t, const char* name) { return const_cast<float*>(f32(t, name)); }
+const int* i32(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kInt && t.is_contiguous(), name, " must be a contiguous int32 GPU tensor");
+  return t.data_ptr<int>();
+}
+// [rows, cols] view with unit column stride (a column slice of a wider projection output)
+int row_stride(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.dim() == 2 && t.stride(1) == 1, name, " must be 2-D with contiguous rows");
+  return (int)t.stride(0);
+}
+
+void add_rmsnorm_f32(Tensor& res, const optional<Tensor>& delta, double mult, const optional<Tensor>& w,
+                     const optional<Tensor>& out, double eps) {
+  float* r = f32w(res, "res");
+  TORCH_CHECK(res.dim() == 2, "add_rmsnorm_f32: res [T, D]");
+  const int T = res.size(0), D = res.size(1);
+  int dd = 0, od = 0, ldd = 0;
+  if (delta) {
+    dd = act_dt(*delta, "delta");
+    ldd = row_stride(*delta, "delta");
+    TORCH_CHECK(delta->size(0) == T && delta->size(1) == D, "add_rmsnorm_f32: delta shape");
+  }
+  if (out) {
+    od = act_dt(*out, "out");
+    TORCH_CHECK(out->is_contiguous() && out->numel() == (int64_t)T * D, "add_rmsnorm_f32: out shape");
+  }
+  TORCH_CHECK(delta || out, "add_rmsnorm_f32: nothing to do");
+  if (w) TORCH_CHECK(w->numel() == D, "add_rmsnorm_f32: weight size");
+  gai_add_rmsnorm_f32(r, delta ? delta->data_ptr() : nullptr, ldd, (float)mult, w ? f32(*w, "w") : nullptr,
+                      out ? out->data_ptr() : nullptr, T, D, (float)eps, dd, od, cur_stream());
+}
+
+void poly_norm(const Tensor& z, const Tensor& coef, double eps, Tensor& y) {
+  const int dt = act_dt(z, "z");
+  same_dt(y, dt, "y");
+  TORCH_CHECK(z.dim() == 2 && z.is_contiguous() && y.is_contiguous() && y.numel() == z.numel(), "poly_norm: shapes");
+  TORCH_CHECK(coef.numel() == 4, "poly_norm: four coefficients");
+  gai_poly_norm(z.data_ptr(), y.data_ptr(), f32(coef, "coef"), z.size(0), z.size(1), (float)eps, dt, cur_stream());
+}
+
+void head_norm_gate(const Tensor& o, const Tensor& gate, const Tensor& nw, int64_t act, double eps, Tensor& y) {
+  TORCH_CHECK(o.dim() == 3, "head_norm_gate: o [T, H, DV]");
+  const int T = o.size(0), H = o.size(1), DV = o.size(2);
+  const int dt = act_dt(gate, "gate");
+  same_dt(y, dt, "y");
+  const int ldg = row_stride(gate, "gate");
+  TORCH_CHECK(gate.size(0) == T && gate.size(1) == H * DV && y.is_contiguous() && y.numel() == o.numel(),
+              "head_norm_gate: gate / y shapes");
+  TORCH_CHECK(nw.numel() == DV || nw.numel() == H * DV, "head_norm_gate: norm weight size");
+  TORCH_CHECK(act == 0 || act == 1, "head_norm_gate: act 0 (silu) or 1 (sigmoid)");
+  gai_head_norm_gate(f32(o, "o"), gate.data_ptr(), ldg, f32(nw, "nw"), nw.numel() == H * DV && H > 1 ? 1 : 0, (int)act,
+                     y.data_ptr(), T, H, DV, (float)eps, dt, cur_stream());
+}
+
+void embed_scale_f32(const Tensor& ids, const Tensor& table, double scale, Tensor& out) {
+  const int dt = act_dt(table, "table");
+  TORCH_CHECK(table.dim() == 2 && table.is_contiguous(), "embed_scale_f32: table [V, D]");
+  const int T = ids.numel(), D = table.size(1);
+  TORCH_CHECK(out.numel() == (int64_t)T * D, "embed_scale_f32: out shape");
+  gai_embed_scale_f32(i32(ids, "ids"), table.data_ptr(), (float)scale, f32w(out, "out"), T, D, table.size(0), dt,
+                      cur_stream());
+}
+
+void check_cache(const Tensor& kc, const Tensor& vc, int dt, int G, int DK, int DV) {
+  same_dt(kc, dt, "k_cache");
+  same_dt(vc, dt, "v_cache");
+  TORCH_CHECK(kc.dim() == 4 && vc.dim() == 4 && kc.is_contiguous() && vc.is_contiguous(), "kv cache: 4-D contiguous");
+  TORCH_CHECK(kc.size(1) == G && kc.size(2) == 16 && kc.size(3) == DK, "k_cache must be [pages, G, 16, DK]");
+  TORCH_CHECK(vc.size(0) == kc.size(0) && vc.size(1) == G && vc.size(2) == DV && vc.size(3) == 16,
+              "v_cache must be [pages, G, DV, 16]");
+}
+
+void qknorm_kv_write(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& wq, const Tensor& wk,
+                     const Tensor& slots, Tensor& q_out, Tensor& k_cache, Tensor& v_cache, int64_t H, int64_t G,
+                     int64_t DK, int64_t DV, double eps) {
+  const int dt = act_dt(q, "q");
+  same_dt(k, dt, "k");
+  same_dt(v, dt, "v");
+  same_dt(q_out, dt, "q_out");
+  check_cache(k_cache, v_cache, dt, G, DK, DV);
+  const int T = q.size(0);
+  TORCH_CHECK(q.size(1) == H * DK && k.size(0) == T && k.size(1) == G * DK && v.size(0) == T && v.size(1) == G * DV,
+              "qknorm_kv_write: projection shapes");
+  TORCH_CHECK(wq.numel() == H * DK && wk.numel() == G * DK && slots.numel() >= T && q_out.is_contiguous() &&
+                  q_out.numel() == (int64_t)T * H * DK, "qknorm_kv_write: weight / slot / output shapes");
+  gai_qknorm_kv_write(q.data_ptr(), row_stride(q, "q"), k.data_ptr(), row_stride(k, "k"), v.data_ptr(),
+                      row_stride(v, "v"), f32(wq, "wq"), f32(wk, "wk"), i32(slots, "slots"), q_out.data_ptr(),
+                      k_cache.data_ptr(), v_cache.data_ptr(), T, H, G, DK, DV, (float)eps, dt, cur_stream());
+}
+
+void window_attention(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& block_tables,
+                      const Tensor& cu_q, const Tensor& ctx, Tensor& out, int64_t H, int64_t G, int64_t DK, int64_t DV,
+                      double scale, double softcap, int64_t window, const optional<Tensor>& r1,
+                      const optional<Tensor>& r2, const optional<Tensor>& gate) {
+  const int dt = act_dt(q, "q");
+  same_dt(out, dt, "out");
+  check_cache(k_cache, v_cache, dt, G, DK, DV);
+  TORCH_CHECK(q.is_contiguous() && out.is_contiguous() && q.numel() % (H * DK) == 0, "window_attention: q shape");
+  const int T = q.numel() / (H * DK);
+  const int S = ctx.numel();
+  TORCH_CHECK(out.numel() == (int64_t)T * H * DV && cu_q.numel() == S + 1 && block_tables.dim() == 2 &&
+                  block_tables.size(0) >= S, "window_attention: out / cu_q / block table shapes");
+  TORCH_CHECK(r1.has_value() == r2.has_value(), "window_attention: r1 and r2 come together");
+  if (r1) TORCH_CHECK(r1->numel() == H && r2->numel() == H, "window_attention: one distance pair per head");
+  int ldg = 0;
+  if (gate) {  // output multiplied by sigmoid(gate), [T, H * DV] rows of a wider projection
+    same_dt(*gate, dt, "gate");
+    ldg = row_stride(*gate, "gate");
+    TORCH_CHECK(gate->size(0) == T && gate->size(1) == H * DV, "window_attention: gate shape");
+  }
+  gai_window_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), i32(block_tables, "block_tables"),
+                       block_tables.size(1), i32(cu_q, "cu_q"), i32(ctx, "ctx"), S, out.data_ptr(), T, H, G, DK, DV,
+                       (float)scale, (float)softcap, (int)window, r1 ? f32(*r1, "r1") : nullptr,
+                       r2 ? f32(*r2, "r2") : nullptr, gate ? gate->data_ptr() : nullptr, ldg, dt, cur_stream());
+}
+
+void token_shift_mix(const Tensor& h, const Tensor& mu, const Tensor& shift_state, const Tensor& cu, const Tensor& slots,
+                     Tensor& out) {
+  const int dt = act_dt(h, "h");
+  same_dt(out, dt, "out");
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && mu.dim() == 2 && mu.size(1) == h.size(1), "token_shift_mix: shapes");
+  const int T = h.size(0), D = h.size(1), NM = mu.size(0), S = slots.numel();
+  TORCH_CHECK(out.is_contiguous() && out.numel() == (int64_t)NM * T * D && cu.numel() == S + 1 &&
+                  shift_state.dim() == 2 && shift_state.size(1) == D, "token_shift_mix: out / cu / state shapes");
+  gai_token_shift_mix(h.data_ptr(), f32(mu, "mu"), NM, f32(shift_state, "shift_state"), i32(cu, "cu"),
+                      i32(slots, "slots"), S, out.data_ptr(), T, D, dt, cur_stream());
+}
+
+void state_tail_write(const Tensor& x, Tensor& state, const Tensor& cu, const Tensor& slots) {
+  const int dt = act_dt(x, "x");
+  const int ldx = row_stride(x, "x");
+  const int C = x.size(1), S = slots.numel();
+  TORCH_CHECK(state.dim() == 3 && state.size(2) == C && cu.numel() == S + 1, "state_tail_write: state [slots, rows, C]");
+  gai_state_tail_write(x.data_ptr(), ldx, f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, C,
+                       (int)state.size(1), dt, cur_stream());
+}
+
+void conv_silu(const Tensor& x, const Tensor& w, const Tensor& state, const Tensor& cu, const Tensor& slots, Tensor& y) {
+  const int dt = act_dt(x, "x");
+  const int ldx = row_stride(x, "x");
+  const int T = x.size(0), C = x.size(1), K = w.size(1), S = slots.numel();
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == C && K >= 1, "conv_silu: weight [C, taps]");
+  TORCH_CHECK(state.dim() == 3 && state.size(1) == K - 1 && state.size(2) == C && cu.numel() == S + 1 &&
+                  y.numel() == (int64_t)T * C, "conv_silu: state / cu / y shapes");
+  gai_conv_silu(x.data_ptr(), ldx, f32(w, "w"), f32(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S,
+                f32w(y, "y"), T, C, K, dt, cur_stream());
+}
+
+void wkv_scan(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& wpre, const Tensor& w0, const Tensor& u,
+              Tensor& state, const Tensor& cu, const Tensor& slots, Tensor& out) {
+  const int dt = act_dt(r, "r");
+  same_dt(k, dt, "k");
+  same_dt(v, dt, "v");
+  TORCH_CHECK(state.dim() == 4 && state.size(2) == state.size(3), "wkv_scan: state [slots, H, D, D]");
+  const int H = state.size(1), D = state.size(2), S = slots.numel();
+  const int ld = row_stride(r, "r");
+  TORCH_CHECK(row_stride(k, "k") == ld && row_stride(v, "v") == ld && r.size(1) == H * D && k.size(1) == H * D &&
+                  v.size(1) == H * D, "wkv_scan: r / k / v must be equal-stride [T, H * D] views");
+  const int T = r.size(0);
+  TORCH_CHECK(k.size(0) == T && v.size(0) == T && wpre.numel() == (int64_t)T * H * D && w0.numel() == H * D &&
+                  u.numel() == H * D && cu.numel() == S + 1 && out.numel() == (int64_t)T * H * D,
+              "wkv_scan: decay / bonus / cu / out shapes");
+  gai_wkv_scan(r.data_ptr(), k.data_ptr(), v.data_ptr(), ld, f32(wpre, "wpre"), f32(w0, "w0"), f32(u, "u"),
+               f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, f32w(out, "out"), H, D, dt, cur_stream());
+}
+
+void delta_prep(const Tensor& qkv, const Tensor& a, const Tensor& b, const Tensor& A_log, const Tensor& dt_bias,
+                Tensor& qn, Tensor& kn, Tensor& decay, Tensor& beta, int64_t H, int64_t G, int64_t DK) {
+  const int dt = act_dt(a, "a");
+  same_dt(b, dt, "b");
+  TORCH_CHECK(qkv.dim() == 2 && qkv.scalar_type() == at::kFloat && qkv.stride(1) == 1 && qkv.size(1) >= 2 * G * DK,
+              "delta_prep: qkv fp32 [T, >= 2 G DK]");
+  const int T = qkv.size(0);
+  TORCH_CHECK(a.size(0) == T && a.size(1) == H * DK && b.size(0) == T && b.size(1) == H && A_log.numel() == H &&
+                  dt_bias.numel() == H * DK, "delta_prep: a / b / A_log / dt_bias shapes");
+  TORCH_CHECK(qn.numel() == (int64_t)T * G * DK && kn.numel() == qn.numel() && decay.numel() == (int64_t)T * H * DK &&
+                  beta.numel() == (int64_t)T * H, "delta_prep: output shapes");
+  gai_delta_prep(qkv.data_ptr<float>(), (int)qkv.stride(0), a.data_ptr(), row_stride(a, "a"), b.data_ptr(),
+                 row_stride(b, "b"), f32(A_log, "A_log"), f32(dt_bias, "dt_bias"), f32w(qn, "qn"), f32w(kn, "kn"),
+                 f32w(decay, "decay"), f32w(beta, "beta"), T, H, G, DK, dt, cur_stream());
+}
+
+void delta_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& decay, const Tensor& beta, Tensor& state,
+                const Tensor& cu, const Tensor& slots, Tensor& out, int64_t G) {
+  TORCH_CHECK(state.dim() == 4, "delta_scan: state [slots, H, DK, DV]");
+  const int H = state.size(1), DK = state.size(2), DV = state.size(3), S = slots.numel();
+  TORCH_CHECK(v.dim() == 2 && v.scalar_type() == at::kFloat && v.stride(1) == 1 && v.size(1) == H * DV,
+              "delta_scan: v fp32 [T, H * DV]");
+  const int T = v.size(0);
+  TORCH_CHECK(q.numel() == (int64_t)T * G * DK && k.numel() == q.numel() && decay.numel() == (int64_t)T * H * DK &&
+                  beta.numel() == (int64_t)T * H && cu.numel() == S + 1 && out.numel() == (int64_t)T * H * DV,
+              "delta_scan: q / k / decay / beta / cu / out shapes");
+  gai_delta_scan(f32(q, "q"), f32(k, "k"), v.data_ptr<float>(), (int)v.stride(0), f32(decay, "decay"), f32(beta, "beta"),
+                 f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, f32w(out, "out"), H, G, DK, DV,
+                 cur_stream());
+}
+
+}  // namespace
+
+void gai_bind_seq_ops(pybind11::module_& m) {
+  m.def("add_rmsnorm_f32", &add_rmsnorm_f32);
+  m.def("poly_norm", &poly_norm);
+  m.def("head_norm_gate", &head_norm_gate);
+  m.def("embed_scale_f32", &embed_scale_f32);
+  m.def("qknorm_kv_write", &qknorm_kv_write);
+  m.def("window_attention", &window_attention);
+  m.def("token_shift_mix", &token_shift_mix);
+  m.def("state_tail_write", &state_tail_write);
+  m.def("conv_silu", &conv_silu);
+  m.def("wkv_scan", &wkv_scan);
+  m.def("delta_prep", &delta_prep);
+  m.def("delta_scan", &delta_scan);
+}

@@ -855,6 +855,8 @@ void gdn_decode(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor&
 
 }  // namespace
 
+void gai_bind_seq_ops(pybind11::module_& m);  // seq_ops.cpp
+
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.doc() = "gfx950 (MI355X) HIP kernels for generativeaiexamples_amd";
   m.def("rmsnorm", &rmsnorm);
@@ -981,5 +983,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
   m.def("ipc_close", [](int64_t p) { gai_ipc_close(reinterpret_cast<void*>(p)); });
   m.attr("AR_CHUNK") = GAI_AR_CHUNK;
   m.attr("AR_MAX_BLOCKS") = GAI_AR_MAX_BLOCKS;
+  gai_bind_seq_ops(m);
   m.attr("ARCH") = "gfx950";
 }

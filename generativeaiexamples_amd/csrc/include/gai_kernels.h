@@ -197,3 +197,38 @@ void gai_gemm_splitk_add_rmsnorm(const void* A, const void* B, const void* bias,
 // gdn.hip (Qwen3-Next gated DeltaNet decode step; state pool [slots, Hv, DK, DV] fp32, updated in place)
 void gai_gdn_decode(const float* q, const float* k, const float* v, const float* g, const float* beta, float* state,
                     const int* slots, float* out, int B, int Hv, int DK, int DV, hipStream_t st);
+
+// ---- sequence mixers with fp32 residual / state (hybrid decoders: window attention, WKV, channel-decay delta rule) ----
+// dt: 0 = bf16 activations, 1 = fp32 activations (weights of the small per-channel tables are always fp32).
+// norm_f32.hip
+void gai_add_rmsnorm_f32(float* res, const void* delta, int ldd, float mult, const float* w, void* out, int T, int D,
+                         float eps, int dt_delta, int dt_out, hipStream_t st);
+void gai_poly_norm(const void* z, void* y, const float* coef, int T, int F, float eps, int dt, hipStream_t st);
+void gai_head_norm_gate(const float* o, const void* gate, int ldg, const float* nw, int nw_per_head, int act, void* y,
+                        int T, int H, int DV, float eps, int dt, hipStream_t st);
+void gai_embed_scale_f32(const int* ids, const void* table, float scale, float* out, int T, int D, int V, int dt,
+                         hipStream_t st);
+// attention_window.hip
+void gai_qknorm_kv_write(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* wq,
+                         const float* wk, const int* slots, void* q_out, void* k_cache, void* v_cache, int T, int H,
+                         int G, int DK, int DV, float eps, int dt, hipStream_t st);
+void gai_window_attention(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int maxb,
+                          const int* cu_q, const int* ctx, int S, void* out, int T, int H, int G, int DK, int DV,
+                          float scale, float softcap, int window, const float* r1, const float* r2, const void* gate,
+                          int ldg, int dt, hipStream_t st);
+// recurrent.hip
+void gai_token_shift_mix(const void* h, const float* mu, int NM, const float* shift_state, const int* cu,
+                         const int* slots, int S, void* out, int T, int D, int dt, hipStream_t st);
+void gai_state_tail_write(const void* x, int ldx, float* state, const int* cu, const int* slots, int S, int C, int NR,
+                          int dt, hipStream_t st);
+void gai_conv_silu(const void* x, int ldx, const float* w, const float* state, const int* cu, const int* slots, int S,
+                   float* y, int T, int C, int K, int dt, hipStream_t st);
+void gai_wkv_scan(const void* r, const void* k, const void* v, int ld, const float* wpre, const float* w0,
+                  const float* u, float* state, const int* cu, const int* slots, int S, float* out, int H, int D,
+                  int dt, hipStream_t st);
+void gai_delta_prep(const float* qkv, int ld, const void* a, int lda, const void* b, int ldb, const float* A_log,
+                    const float* dt_bias, float* qn, float* kn, float* decay, float* beta, int T, int H, int G, int DK,
+                    int dt, hipStream_t st);
+void gai_delta_scan(const float* q, const float* k, const float* v, int ldv, const float* decay, const float* beta,
+                    float* state, const int* cu, const int* slots, int S, float* out, int H, int G, int DK, int DV,
+                    hipStream_t st);

@@ -1,0 +1,234 @@
+// Sliding-window paged attention with a tanh score cap and a logarithmic distance penalty, in fp32 arithmetic.
+//
+//   s_ij = cap * tanh(scale * (q_i . k_j) / cap) - r1_h * ln(1 + r2_h * (i - j)),   0 <= i - j < window
+//   o_i  = softmax_j(s_ij) V
+//
+// optionally times sigmoid(gate_i) element by element (an output gate read from the same projection as q, k, v).
+// (cap <= 0: no cap; r1 = nullptr: no distance term; window <= 0: plain causal.) Positions enter only through the
+// distance term and the window: there is no rotation. K / V live in the engine's paged cache (16-token pages,
+// K [page, G, 16, DK], V^T [page, G, DV, 16]) in bf16 or fp32; scores, softmax weights and the P.V sums are fp32.
+// Head sizes are run-time values (DK != DV allowed, DV <= 256).
+//
+// qknorm_kv_write: RMS norm over the WHOLE q projection (all heads at once) and over the whole k projection, each
+// with its own weight vector, then q -> q_out and k, v -> their cache slots: one pass over the token's rows.
+//
+// window_attention: one wave64 per (token, head), for prompt portions and single decoded tokens alike (a sequence is
+// (cu_q[s], ctx[s]); the query at row t has position ctx - q_len + (t - cu_q)). Keys are walked in page-aligned
+// blocks of 64: lane j scores key j (q broadcast from LDS, the K row read with 16-byte loads), an online softmax
+// keeps (m, l) per wave, then lane c accumulates output channel c over the block, reading its 16 V^T values of every
+// page with 16-byte loads.
+#include "gai_common.h"
+#include "gai_kernels.h"
+
+using namespace gai;
+
+namespace {
+
+__device__ __forceinline__ float dot_row(const float* __restrict__ qs, const bf16* __restrict__ k, int DK) {
+  float a = 0.f;
+  if ((DK & 7) == 0) {
+    for (int i = 0; i < DK; i += 8) {
+      const bf16x8 v = load8(k + i);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) a = fmaf(qs[i + j], (float)v[j], a);
+    }
+  } else {
+    for (int i = 0; i < DK; ++i) a = fmaf(qs[i], (float)k[i], a);
+  }
+  return a;
+}
+
+__device__ __forceinline__ float dot_row(const float* __restrict__ qs, const float* __restrict__ k, int DK) {
+  float a = 0.f;
+  if ((DK & 3) == 0) {
+    for (int i = 0; i < DK; i += 4) {
+      const float4 v = *reinterpret_cast<const float4*>(k + i);
+      a = fmaf(qs[i], v.x, a);
+      a = fmaf(qs[i + 1], v.y, a);
+      a = fmaf(qs[i + 2], v.z, a);
+      a = fmaf(qs[i + 3], v.w, a);
+    }
+  } else {
+    for (int i = 0; i < DK; ++i) a = fmaf(qs[i], k[i], a);
+  }
+  return a;
+}
+
+// sum_j p[j] * v[j] over the 16 tokens of one V^T page row
+__device__ __forceinline__ float pv16(const float* __restrict__ p, const bf16* __restrict__ v) {
+  const bf16x8 a = load8(v), b = load8(v + 8);
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s = fmaf(p[j], (float)a[j], s);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) s = fmaf(p[8 + j], (float)b[j], s);
+  return s;
+}
+
+__device__ __forceinline__ float pv16(const float* __restrict__ p, const float* __restrict__ v) {
+  float s = 0.f;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const float4 a = *reinterpret_cast<const float4*>(v + 4 * q);
+    s = fmaf(p[4 * q], a.x, s);
+    s = fmaf(p[4 * q + 1], a.y, s);
+    s = fmaf(p[4 * q + 2], a.z, s);
+    s = fmaf(p[4 * q + 3], a.w, s);
+  }
+  return s;
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void qknorm_kv_write_kernel(const TA* __restrict__ q, int ldq, const TA* __restrict__ k,
+                                                              int ldk, const TA* __restrict__ v, int ldv,
+                                                              const float* __restrict__ wq, const float* __restrict__ wk,
+                                                              const int* __restrict__ slots, TA* __restrict__ q_out,
+                                                              TA* __restrict__ k_cache, TA* __restrict__ v_cache, int H,
+                                                              int G, int DK, int DV, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const TA* qr = q + (size_t)t * ldq;
+  const TA* kr = k + (size_t)t * ldk;
+  const TA* vr = v + (size_t)t * ldv;
+  const int NQ = H * DK, NK = G * DK, NV = G * DV;
+  float sq = 0.f, sk = 0.f;
+  for (int i = tid; i < NQ; i += 256) {
+    const float x = (float)qr[i];
+    sq += x * x;
+  }
+  for (int i = tid; i < NK; i += 256) {
+    const float x = (float)kr[i];
+    sk += x * x;
+  }
+  sq = block_sum(sq, scratch);
+  sk = block_sum(sk, scratch);
+  const float iq = 1.0f / sqrtf(sq / NQ + eps), ik = 1.0f / sqrtf(sk / NK + eps);
+  TA* qo = q_out + (size_t)t * NQ;
+  for (int i = tid; i < NQ; i += 256) qo[i] = (TA)((float)qr[i] * iq * wq[i]);
+  const int slot = slots[t];
+  const size_t page = slot >> 4;
+  const int off = slot & 15;
+  for (int i = tid; i < NK; i += 256) {
+    const int g = i / DK, d = i - g * DK;
+    k_cache[((page * G + g) * 16 + off) * DK + d] = (TA)((float)kr[i] * ik * wk[i]);
+  }
+  for (int i = tid; i < NV; i += 256) {
+    const int g = i / DV, c = i - g * DV;
+    v_cache[((page * G + g) * DV + c) * 16 + off] = vr[i];
+  }
+}
+
+constexpr int kMaxVChunks = 4;  // DV <= 256
+
+template <typename TA>
+__global__ __launch_bounds__(256) void window_attention_kernel(
+    const TA* __restrict__ q, const TA* __restrict__ k_cache, const TA* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int maxb, const int* __restrict__ cu_q, const int* __restrict__ ctx, int S,
+    TA* __restrict__ out, int TH, int H, int G, int DK, int DV, float scale, float softcap, int window,
+    const float* __restrict__ r1, const float* __restrict__ r2, const TA* __restrict__ gate, int ldg) {
+  extern __shared__ float lds[];
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int th = blockIdx.x * 4 + wid;
+  if (th >= TH) return;  // wave-uniform; no workgroup barrier below
+  float* qs = lds + wid * (DK + 64);
+  float* ps = qs + DK;
+  const int t = th / H, h = th - t * H, g = h / (H / G);
+  int lo = 0, hi = S;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu_q[mid] <= t) lo = mid; else hi = mid;
+  }
+  const int s = lo, c0 = cu_q[s];
+  const int pos = ctx[s] - (cu_q[s + 1] - c0) + (t - c0);
+  const int first = window > 0 ? max(0, pos - window + 1) : 0;
+  const TA* qr = q + (size_t)th * DK;
+  for (int i = lane; i < DK; i += 64) qs[i] = (float)qr[i];
+  __builtin_amdgcn_wave_barrier();
+  const float b1 = r1 ? r1[h] : 0.f, b2 = r1 ? r2[h] : 0.f;
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+  const int* bt = block_tables + (size_t)s * maxb;
+  float m = -INFINITY, l = 0.f, acc[kMaxVChunks];
+#pragma unroll
+  for (int n = 0; n < kMaxVChunks; ++n) acc[n] = 0.f;
+  for (int kb = first & ~15; kb <= pos; kb += 64) {
+    const int p = kb + lane;
+    const bool valid = p >= first && p <= pos;
+    float sc = -INFINITY;
+    if (valid) {
+      const size_t page = bt[p >> 4];
+      sc = dot_row(qs, k_cache + ((page * G + g) * 16 + (p & 15)) * DK, DK) * scale;
+      if (softcap > 0.f) sc = softcap * tanhf(sc * inv_cap);
+      if (r1) sc -= b1 * log1pf(b2 * (float)(pos - p));
+    }
+    const float m_new = fmaxf(m, wave_max(sc));
+    const float pe = valid ? expf(sc - m_new) : 0.f;
+    const float alpha = expf(m - m_new);
+    l = l * alpha + wave_sum(pe);
+    m = m_new;
+    __builtin_amdgcn_wave_barrier();  // the previous block's reads of ps are done
+    ps[lane] = pe;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int n = 0; n < kMaxVChunks; ++n) acc[n] *= alpha;
+    for (int pg = 0; pg < 4; ++pg) {
+      const int pp = kb + 16 * pg;
+      if (pp > pos) break;
+      if (pp + 15 < first) continue;
+      const size_t page = bt[pp >> 4];
+#pragma unroll
+      for (int n = 0; n < kMaxVChunks; ++n) {
+        const int c = lane + 64 * n;
+        if (c < DV) acc[n] += pv16(ps + 16 * pg, v_cache + ((page * G + g) * DV + c) * 16);
+      }
+    }
+  }
+  const float inv_l = 1.0f / l;
+  TA* o = out + (size_t)th * DV;
+#pragma unroll
+  for (int n = 0; n < kMaxVChunks; ++n) {
+    const int c = lane + 64 * n;
+    if (c < DV) {
+      float y = acc[n] * inv_l;
+      if (gate) y *= 1.0f / (1.0f + expf(-(float)gate[(size_t)t * ldg + (size_t)h * DV + c]));
+      o[c] = (TA)y;
+    }
+  }
+}
+
+}  // namespace
+
+void gai_qknorm_kv_write(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* wq,
+                         const float* wk, const int* slots, void* q_out, void* k_cache, void* v_cache, int T, int H,
+                         int G, int DK, int DV, float eps, int dt, hipStream_t st) {
+  if (T == 0) return;
+  if (dt)
+    qknorm_kv_write_kernel<float><<<T, 256, 0, st>>>((const float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv, wq,
+                                                     wk, slots, (float*)q_out, (float*)k_cache, (float*)v_cache, H, G,
+                                                     DK, DV, eps);
+  else
+    qknorm_kv_write_kernel<bf16><<<T, 256, 0, st>>>((const bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv, wq, wk,
+                                                    slots, (bf16*)q_out, (bf16*)k_cache, (bf16*)v_cache, H, G, DK, DV,
+                                                    eps);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_window_attention(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int maxb,
+                          const int* cu_q, const int* ctx, int S, void* out, int T, int H, int G, int DK, int DV,
+                          float scale, float softcap, int window, const float* r1, const float* r2, const void* gate,
+                          int ldg, int dt, hipStream_t st) {
+  if (T == 0 || S == 0) return;
+  if (DV > 64 * kMaxVChunks) gai_launch_error(__FILE__, __LINE__, "window_attention: value head size above 256");
+  if (H % G) gai_launch_error(__FILE__, __LINE__, "window_attention: heads must be a multiple of kv heads");
+  const int TH = T * H, grid = (TH + 3) / 4;
+  const size_t lds = 4 * (size_t)(DK + 64) * sizeof(float);
+  if (dt)
+    window_attention_kernel<float><<<grid, 256, lds, st>>>((const float*)q, (const float*)k_cache,
+                                                           (const float*)v_cache, block_tables, maxb, cu_q, ctx, S,
+                                                           (float*)out, TH, H, G, DK, DV, scale, softcap, window, r1, r2,
+                                                           (const float*)gate, ldg);
+  else
+    window_attention_kernel<bf16><<<grid, 256, lds, st>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache,
+                                                          block_tables, maxb, cu_q, ctx, S, (bf16*)out, TH, H, G, DK,
+                                                          DV, scale, softcap, window, r1, r2, (const bf16*)gate, ldg);
+  GAI_LAUNCH_CHECK();
+}

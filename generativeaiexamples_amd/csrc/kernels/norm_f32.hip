@@ -1,0 +1,160 @@
+// Normalisations around a 32-bit residual stream (hybrid decoders whose residual sum, norms and recurrent
+// inputs stay in fp32 while the matrix products run in bf16).
+//
+//   add_rmsnorm_f32   res += mult * delta;  out = res * rsqrt(mean(res^2) + eps) * w      (w = nullptr: out = res)
+//   poly_norm         y = a N(z) + b N(z^2) + c N(z^3) + e,  N(t) = t * rsqrt(mean(t^2) + eps) over the row
+//   head_norm_gate    y = o * rsqrt(mean_head(o^2) + eps) * nw * act(gate)   (act: silu | sigmoid), one head per wave
+//   embed_scale_f32   out = table[id] * scale as fp32
+//
+// Activations (delta, z, gate, out, y) are bf16 or fp32 (template TA); every statistic and product is fp32.
+// One wave64 per row for the row norms (D of a few thousand: the row is re-read from L2 in the second pass).
+#include "gai_common.h"
+#include "gai_kernels.h"
+
+using namespace gai;
+
+namespace {
+
+template <typename TD, typename TA>
+__global__ __launch_bounds__(256) void add_rmsnorm_f32_kernel(float* __restrict__ res, const TD* __restrict__ delta,
+                                                              int ldd, float mult, const float* __restrict__ w,
+                                                              TA* __restrict__ out, int T, int D, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= T) return;
+  float* r = res + (size_t)row * D;
+  float s = 0.f;
+  if (delta) {
+    const TD* d = delta + (size_t)row * ldd;
+    for (int i = lane; i < D; i += 64) {
+      const float v = r[i] + mult * (float)d[i];
+      r[i] = v;
+      s += v * v;
+    }
+  } else {
+    for (int i = lane; i < D; i += 64) {
+      const float v = r[i];
+      s += v * v;
+    }
+  }
+  if (!out) return;
+  TA* o = out + (size_t)row * D;
+  if (!w) {
+    for (int i = lane; i < D; i += 64) o[i] = (TA)r[i];
+    return;
+  }
+  s = wave_sum(s);
+  const float inv = 1.0f / sqrtf(s / D + eps);
+  for (int i = lane; i < D; i += 64) o[i] = (TA)(r[i] * inv * w[i]);
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void poly_norm_kernel(const TA* __restrict__ z, TA* __restrict__ y,
+                                                        const float* __restrict__ coef, int F, float eps) {
+  __shared__ float scratch[16];
+  const TA* zr = z + (size_t)blockIdx.x * F;
+  TA* yr = y + (size_t)blockIdx.x * F;
+  float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  for (int i = threadIdx.x; i < F; i += 256) {
+    const float v = (float)zr[i], v2 = v * v;
+    s1 += v2;
+    s2 += v2 * v2;
+    s3 += v2 * v2 * v2;
+  }
+  s1 = block_sum(s1, scratch);
+  s2 = block_sum(s2, scratch);
+  s3 = block_sum(s3, scratch);
+  const float a = coef[0] / sqrtf(s1 / F + eps), b = coef[1] / sqrtf(s2 / F + eps), c = coef[2] / sqrtf(s3 / F + eps);
+  const float e = coef[3];
+  for (int i = threadIdx.x; i < F; i += 256) {
+    const float v = (float)zr[i];
+    yr[i] = (TA)(a * v + b * v * v + c * v * v * v + e);
+  }
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const TA* __restrict__ gate,
+                                                             int ldg, const float* __restrict__ nw, int nw_per_head,
+                                                             int act, TA* __restrict__ y, int TH, int H, int DV,
+                                                             float eps) {
+  const int lane = threadIdx.x & 63;
+  const int th = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (th >= TH) return;
+  const int t = th / H, h = th % H;
+  const float* orow = o + (size_t)th * DV;
+  float s = 0.f;
+  for (int i = lane; i < DV; i += 64) s += orow[i] * orow[i];
+  s = wave_sum(s);
+  const float inv = 1.0f / sqrtf(s / DV + eps);
+  const TA* g = gate + (size_t)t * ldg + (size_t)h * DV;
+  const float* wr = nw + (nw_per_head ? (size_t)h * DV : 0);
+  TA* yr = y + (size_t)th * DV;
+  for (int i = lane; i < DV; i += 64) {
+    const float gv = (float)g[i];
+    const float sg = 1.0f / (1.0f + expf(-gv));
+    yr[i] = (TA)(orow[i] * inv * wr[i] * (act == 0 ? gv * sg : sg));
+  }
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void embed_scale_f32_kernel(const int* __restrict__ ids, const TA* __restrict__ table,
+                                                              float scale, float* __restrict__ out, int T, int D,
+                                                              int V) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= T) return;
+  int id = ids[row];
+  id = id < 0 ? 0 : (id >= V ? V - 1 : id);
+  const TA* e = table + (size_t)id * D;
+  float* o = out + (size_t)row * D;
+  for (int i = lane; i < D; i += 64) o[i] = (float)e[i] * scale;
+}
+
+}  // namespace
+
+void gai_add_rmsnorm_f32(float* res, const void* delta, int ldd, float mult, const float* w, void* out, int T, int D,
+                         float eps, int dt_delta, int dt_out, hipStream_t st) {
+  if (T == 0) return;
+  const int grid = (T + 3) / 4;
+#define GAI_ARN(TD, TA) \
+  add_rmsnorm_f32_kernel<TD, TA><<<grid, 256, 0, st>>>(res, (const TD*)delta, ldd, mult, w, (TA*)out, T, D, eps)
+  if (dt_delta && dt_out) GAI_ARN(float, float);
+  else if (dt_delta) GAI_ARN(float, bf16);
+  else if (dt_out) GAI_ARN(bf16, float);
+  else GAI_ARN(bf16, bf16);
+#undef GAI_ARN
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_poly_norm(const void* z, void* y, const float* coef, int T, int F, float eps, int dt, hipStream_t st) {
+  if (T == 0) return;
+  if (dt)
+    poly_norm_kernel<float><<<T, 256, 0, st>>>((const float*)z, (float*)y, coef, F, eps);
+  else
+    poly_norm_kernel<bf16><<<T, 256, 0, st>>>((const bf16*)z, (bf16*)y, coef, F, eps);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_head_norm_gate(const float* o, const void* gate, int ldg, const float* nw, int nw_per_head, int act, void* y,
+                        int T, int H, int DV, float eps, int dt, hipStream_t st) {
+  if (T == 0) return;
+  const int TH = T * H, grid = (TH + 3) / 4;
+  if (dt)
+    head_norm_gate_kernel<float><<<grid, 256, 0, st>>>(o, (const float*)gate, ldg, nw, nw_per_head, act, (float*)y, TH,
+                                                        H, DV, eps);
+  else
+    head_norm_gate_kernel<bf16><<<grid, 256, 0, st>>>(o, (const bf16*)gate, ldg, nw, nw_per_head, act, (bf16*)y, TH, H,
+                                                       DV, eps);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_embed_scale_f32(const int* ids, const void* table, float scale, float* out, int T, int D, int V, int dt,
+                         hipStream_t st) {
+  if (T == 0) return;
+  const int grid = (T + 3) / 4;
+  if (dt)
+    embed_scale_f32_kernel<float><<<grid, 256, 0, st>>>(ids, (const float*)table, scale, out, T, D, V);
+  else
+    embed_scale_f32_kernel<bf16><<<grid, 256, 0, st>>>(ids, (const bf16*)table, scale, out, T, D, V);
+  GAI_LAUNCH_CHECK();
+}

@@ -1,0 +1,333 @@
+// Recurrent sequence mixers over a per-sequence fp32 state pool (slot = one live sequence):
+//
+//   token_shift_mix   m_s[t] = h[t] + (h[t-1] - h[t]) * mu_s   for NM mixes; h[-1] of a portion comes from the pool
+//   conv_silu         short causal depthwise convolution over time (last tap = current token) + SiLU; the inputs before
+//                     a portion's first token come from the pool (zeros for a fresh sequence)
+//   state_tail_write  keep the last NR input rows of every sequence in the pool (token shift: NR = 1; conv: taps - 1)
+//   wkv_scan          S [DK, DV] per head:  o_t = (S + diag(u) k_t v_t^T)^T r_t;  S <- diag(w_t) S + k_t v_t^T,
+//                     w_t = exp(-exp(wpre_t + w0))
+//   delta_prep        token-parallel inputs of the delta rule: unit-norm q (x DK^-1/2) and k per head, per-channel
+//                     decay exp(-exp(A_log_h) softplus(a + dt_bias)), write strength sigmoid(b)
+//   delta_scan        S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
+//
+// A batch is S sequences of rows [cu[s], cu[s+1]) with pool slot slots[s] (device vectors: graph-capturable); a decoded
+// token is a sequence of one row, a prompt portion a longer one, and the same kernels run both. The scans keep the
+// state in VGPRs for the whole portion: one workgroup per (head, sequence), thread (rg, j) owns rows [64 rg, 64 rg + 64)
+// of state column j, token inputs are double-buffered in LDS (two barriers per token, three when the delta rule needs
+// its read-before-write reduction across row groups), and the state is read from / written to the pool once.
+#include "gai_common.h"
+#include "gai_kernels.h"
+
+using namespace gai;
+
+namespace {
+
+constexpr int kRows = 64;     // state rows per thread
+constexpr int kMaxRG = 4;     // DK <= 256
+constexpr int kMaxDK = kRows * kMaxRG;
+
+template <typename TA>
+__global__ __launch_bounds__(256) void token_shift_mix_kernel(const TA* __restrict__ h, const float* __restrict__ mu,
+                                                              int NM, const float* __restrict__ shift_state,
+                                                              const int* __restrict__ cu, const int* __restrict__ slots,
+                                                              int S, TA* __restrict__ out, int T, int D) {
+  const int t = blockIdx.x;
+  int lo = 0, hi = S;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu[mid] <= t) lo = mid; else hi = mid;
+  }
+  const bool head = cu[lo] == t;
+  const float* prev_s = shift_state + (size_t)slots[lo] * D;
+  const TA* cur = h + (size_t)t * D;
+  for (int i = threadIdx.x; i < D; i += 256) {
+    const float x = (float)cur[i];
+    const float xp = head ? prev_s[i] : (float)cur[i - D];
+    const float d = xp - x;
+    for (int n = 0; n < NM; ++n) out[((size_t)n * T + t) * D + i] = (TA)(x + d * mu[(size_t)n * D + i]);
+  }
+}
+
+// One thread per (sequence, channel): read every value the new tail needs, then write (the tail may overlap itself).
+template <typename TA>
+__global__ __launch_bounds__(256) void state_tail_write_kernel(const TA* __restrict__ x, int ldx, float* __restrict__ state,
+                                                               const int* __restrict__ cu, const int* __restrict__ slots,
+                                                               int C, int NR) {
+  const int s = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int b = cu[s], L = cu[s + 1] - b;
+  if (L <= 0) return;
+  float* st = state + (size_t)slots[s] * NR * C + c;
+  float keep[8];
+#pragma unroll
+  for (int r = 0; r < 8; ++r) {
+    if (r < NR) {
+      const int src = L - NR + r;  // row of the portion; negative: older, from the pool
+      keep[r] = src >= 0 ? (float)x[(size_t)(b + src) * ldx + c] : st[(size_t)(NR + src) * C];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 8; ++r)
+    if (r < NR) st[(size_t)r * C] = keep[r];
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void conv_silu_kernel(const TA* __restrict__ x, int ldx, const float* __restrict__ w,
+                                                        const float* __restrict__ state, const int* __restrict__ cu,
+                                                        const int* __restrict__ slots, int S, float* __restrict__ y,
+                                                        int C, int K) {
+  const int t = blockIdx.x;
+  int lo = 0, hi = S;
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (cu[mid] <= t) lo = mid; else hi = mid;
+  }
+  const int rel = t - cu[lo];
+  const float* st = state + (size_t)slots[lo] * (K - 1) * C;
+  for (int c = threadIdx.x; c < C; c += 256) {
+    float a = 0.f;
+    for (int i = 0; i < K; ++i) {
+      const int src = rel - (K - 1) + i;
+      const float xv = src >= 0 ? (float)x[(size_t)(t - (K - 1) + i) * ldx + c] : st[(size_t)(K - 1 + src) * C + c];
+      a = fmaf(xv, w[(size_t)c * K + i], a);
+    }
+    y[(size_t)t * C + c] = a / (1.0f + expf(-a));
+  }
+}
+
+template <typename TA>
+__global__ __launch_bounds__(1024) void wkv_scan_kernel(const TA* __restrict__ r, const TA* __restrict__ k,
+                                                        const TA* __restrict__ v, int ld, const float* __restrict__ wpre,
+                                                        const float* __restrict__ w0, const float* __restrict__ u,
+                                                        float* __restrict__ state, const int* __restrict__ cu,
+                                                        const int* __restrict__ slots, float* __restrict__ out, int H,
+                                                        int D) {
+  extern __shared__ float lds[];  // us[D] | buf[2][3][D] (r, k, w) | red[2][RG][D]
+  const int h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
+  const int RG = (D + kRows - 1) / kRows;
+  const int j = tid % D, rg = tid / D;
+  const int row0 = rg * kRows, nrow = min(kRows, D - row0);
+  float* us = lds;
+  float* buf = us + D;
+  float* red = buf + 6 * D;
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;
+  float* Sg = state + (((size_t)slots[s] * H + h) * D + row0) * D + j;
+  float col[kRows];
+#pragma unroll
+  for (int i = 0; i < kRows; ++i) col[i] = i < nrow ? Sg[(size_t)i * D] : 0.f;
+  if (tid < D) us[tid] = u[(size_t)h * D + tid];
+  for (int t = t0; t < t1; ++t) {
+    const int b = (t - t0) & 1;
+    float* rb = buf + b * 3 * D;
+    if (tid < D) {
+      const size_t o = (size_t)t * ld + (size_t)h * D + tid;
+      rb[tid] = (float)r[o];
+      rb[D + tid] = (float)k[o];
+      rb[2 * D + tid] = expf(-expf(wpre[((size_t)t * H + h) * D + tid] + w0[(size_t)h * D + tid]));
+    }
+    const float vj = (float)v[(size_t)t * ld + (size_t)h * D + j];
+    __syncthreads();
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < kRows; ++i) {
+      if (i < nrow) {
+        const float kv = rb[D + row0 + i] * vj;
+        acc = fmaf(rb[row0 + i], fmaf(us[row0 + i], kv, col[i]), acc);
+        col[i] = fmaf(rb[2 * D + row0 + i], col[i], kv);
+      }
+    }
+    if (RG == 1) {
+      out[((size_t)t * H + h) * D + j] = acc;
+    } else {
+      red[(b * RG + rg) * D + j] = acc;
+      __syncthreads();
+      if (rg == 0) {
+        float o = 0.f;
+        for (int g = 0; g < RG; ++g) o += red[(b * RG + g) * D + j];
+        out[((size_t)t * H + h) * D + j] = o;
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kRows; ++i)
+    if (i < nrow) Sg[(size_t)i * D] = col[i];
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void delta_prep_kernel(const float* __restrict__ qkv, int ld, const TA* __restrict__ a,
+                                                         int lda, const TA* __restrict__ bp, int ldb,
+                                                         const float* __restrict__ A_log, const float* __restrict__ dt_bias,
+                                                         float* __restrict__ qn, float* __restrict__ kn,
+                                                         float* __restrict__ decay, float* __restrict__ beta, int H, int G,
+                                                         int DK) {
+  const int t = blockIdx.x, wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const float* row = qkv + (size_t)t * ld;
+  const float qscale = 1.0f / sqrtf((float)DK);
+  for (int gh = wid; gh < 2 * G; gh += 4) {  // q heads then k heads
+    const float* src = row + (size_t)gh * DK;
+    float s = 0.f;
+    for (int i = lane; i < DK; i += 64) s += src[i] * src[i];
+    s = wave_sum(s);
+    const float inv = (1.0f / sqrtf(s + 1e-6f)) * (gh < G ? qscale : 1.0f);
+    float* dst = gh < G ? qn + ((size_t)t * G + gh) * DK : kn + ((size_t)t * G + (gh - G)) * DK;
+    for (int i = lane; i < DK; i += 64) dst[i] = src[i] * inv;
+  }
+  const int HD = H * DK;
+  for (int i = threadIdx.x; i < HD; i += 256) {
+    const float x = (float)a[(size_t)t * lda + i] + dt_bias[i];
+    const float sp = x > 20.f ? x : log1pf(expf(x));
+    decay[(size_t)t * HD + i] = expf(-expf(A_log[i / DK]) * sp);
+  }
+  for (int i = threadIdx.x; i < H; i += 256) beta[(size_t)t * H + i] = 1.0f / (1.0f + expf(-(float)bp[(size_t)t * ldb + i]));
+}
+
+__global__ __launch_bounds__(1024) void delta_scan_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                          const float* __restrict__ v, int ldv,
+                                                          const float* __restrict__ decay, const float* __restrict__ beta,
+                                                          float* __restrict__ state, const int* __restrict__ cu,
+                                                          const int* __restrict__ slots, float* __restrict__ out, int H,
+                                                          int G, int DK, int DV) {
+  extern __shared__ float lds[];  // buf[2][3][DK] (q, k, g) | red[2][2][RG][DV]
+  const int h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
+  const int RG = (DK + kRows - 1) / kRows;
+  const int j = tid % DV, rg = tid / DV;
+  const int row0 = rg * kRows, nrow = min(kRows, DK - row0);
+  const int g = h / (H / G);
+  float* buf = lds;
+  float* red = buf + 6 * DK;
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;
+  float* Sg = state + (((size_t)slots[s] * H + h) * DK + row0) * DV + j;
+  float col[kRows];
+#pragma unroll
+  for (int i = 0; i < kRows; ++i) col[i] = i < nrow ? Sg[(size_t)i * DV] : 0.f;
+  for (int t = t0; t < t1; ++t) {
+    const int b = (t - t0) & 1;
+    float* qb = buf + b * 3 * DK;
+    for (int i = tid; i < DK; i += blockDim.x) {
+      qb[i] = q[((size_t)t * G + g) * DK + i];
+      qb[DK + i] = k[((size_t)t * G + g) * DK + i];
+      qb[2 * DK + i] = decay[((size_t)t * H + h) * DK + i];
+    }
+    const float vj = v[(size_t)t * ldv + (size_t)h * DV + j];
+    const float bt = beta[(size_t)t * H + h];
+    __syncthreads();
+    float mm = 0.f;
+#pragma unroll
+    for (int i = 0; i < kRows; ++i) {
+      if (i < nrow) {
+        col[i] *= qb[2 * DK + row0 + i];
+        mm = fmaf(col[i], qb[DK + row0 + i], mm);
+      }
+    }
+    if (RG > 1) {
+      float* rm = red + ((b * 2 + 0) * RG) * DV;
+      rm[rg * DV + j] = mm;
+      __syncthreads();
+      mm = 0.f;
+      for (int x = 0; x < RG; ++x) mm += rm[x * DV + j];
+    }
+    const float uj = bt * (vj - mm);
+    float oo = 0.f;
+#pragma unroll
+    for (int i = 0; i < kRows; ++i) {
+      if (i < nrow) {
+        col[i] = fmaf(qb[DK + row0 + i], uj, col[i]);
+        oo = fmaf(col[i], qb[row0 + i], oo);
+      }
+    }
+    if (RG == 1) {
+      out[((size_t)t * H + h) * DV + j] = oo;
+    } else {
+      float* ro = red + ((b * 2 + 1) * RG) * DV;
+      ro[rg * DV + j] = oo;
+      __syncthreads();
+      if (rg == 0) {
+        float o = 0.f;
+        for (int x = 0; x < RG; ++x) o += ro[x * DV + j];
+        out[((size_t)t * H + h) * DV + j] = o;
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kRows; ++i)
+    if (i < nrow) Sg[(size_t)i * DV] = col[i];
+}
+
+}  // namespace
+
+void gai_token_shift_mix(const void* h, const float* mu, int NM, const float* shift_state, const int* cu,
+                         const int* slots, int S, void* out, int T, int D, int dt, hipStream_t st) {
+  if (T == 0) return;
+  if (dt)
+    token_shift_mix_kernel<float><<<T, 256, 0, st>>>((const float*)h, mu, NM, shift_state, cu, slots, S, (float*)out, T, D);
+  else
+    token_shift_mix_kernel<bf16><<<T, 256, 0, st>>>((const bf16*)h, mu, NM, shift_state, cu, slots, S, (bf16*)out, T, D);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_state_tail_write(const void* x, int ldx, float* state, const int* cu, const int* slots, int S, int C, int NR,
+                          int dt, hipStream_t st) {
+  if (S == 0 || NR == 0) return;
+  if (NR > 8) gai_launch_error(__FILE__, __LINE__, "state_tail_write: more than 8 rows kept");
+  const dim3 grid((C + 255) / 256, S);
+  if (dt)
+    state_tail_write_kernel<float><<<grid, 256, 0, st>>>((const float*)x, ldx, state, cu, slots, C, NR);
+  else
+    state_tail_write_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, ldx, state, cu, slots, C, NR);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_conv_silu(const void* x, int ldx, const float* w, const float* state, const int* cu, const int* slots, int S,
+                   float* y, int T, int C, int K, int dt, hipStream_t st) {
+  if (T == 0) return;
+  if (dt)
+    conv_silu_kernel<float><<<T, 256, 0, st>>>((const float*)x, ldx, w, state, cu, slots, S, y, C, K);
+  else
+    conv_silu_kernel<bf16><<<T, 256, 0, st>>>((const bf16*)x, ldx, w, state, cu, slots, S, y, C, K);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_wkv_scan(const void* r, const void* k, const void* v, int ld, const float* wpre, const float* w0,
+                  const float* u, float* state, const int* cu, const int* slots, int S, float* out, int H, int D,
+                  int dt, hipStream_t st) {
+  if (S == 0) return;
+  const int RG = (D + kRows - 1) / kRows;
+  if (D > kMaxDK || D * RG > 1024) gai_launch_error(__FILE__, __LINE__, "wkv_scan: head size above 256");
+  const dim3 grid(H, S);
+  const size_t lds = (size_t)(7 * D + 2 * RG * D) * sizeof(float);
+  if (dt)
+    wkv_scan_kernel<float><<<grid, D * RG, lds, st>>>((const float*)r, (const float*)k, (const float*)v, ld, wpre, w0, u,
+                                                      state, cu, slots, out, H, D);
+  else
+    wkv_scan_kernel<bf16><<<grid, D * RG, lds, st>>>((const bf16*)r, (const bf16*)k, (const bf16*)v, ld, wpre, w0, u,
+                                                     state, cu, slots, out, H, D);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_delta_prep(const float* qkv, int ld, const void* a, int lda, const void* b, int ldb, const float* A_log,
+                    const float* dt_bias, float* qn, float* kn, float* decay, float* beta, int T, int H, int G, int DK,
+                    int dt, hipStream_t st) {
+  if (T == 0) return;
+  if (dt)
+    delta_prep_kernel<float><<<T, 256, 0, st>>>(qkv, ld, (const float*)a, lda, (const float*)b, ldb, A_log, dt_bias, qn,
+                                                kn, decay, beta, H, G, DK);
+  else
+    delta_prep_kernel<bf16><<<T, 256, 0, st>>>(qkv, ld, (const bf16*)a, lda, (const bf16*)b, ldb, A_log, dt_bias, qn, kn,
+                                               decay, beta, H, G, DK);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_delta_scan(const float* q, const float* k, const float* v, int ldv, const float* decay, const float* beta,
+                    float* state, const int* cu, const int* slots, int S, float* out, int H, int G, int DK, int DV,
+                    hipStream_t st) {
+  if (S == 0) return;
+  const int RG = (DK + kRows - 1) / kRows;
+  if (DK > kMaxDK || DV * RG > 1024) gai_launch_error(__FILE__, __LINE__, "delta_scan: head sizes above 256");
+  if (H % G) gai_launch_error(__FILE__, __LINE__, "delta_scan: heads must be a multiple of key heads");
+  const dim3 grid(H, S);
+  const size_t lds = (size_t)(6 * DK + 4 * RG * DV) * sizeof(float);
+  delta_scan_kernel<<<grid, DV * RG, lds, st>>>(q, k, v, ldv, decay, beta, state, cu, slots, out, H, G, DK, DV);
+  GAI_LAUNCH_CHECK();
+}

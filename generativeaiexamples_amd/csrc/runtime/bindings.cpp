@@ -103,6 +103,8 @@ PYBIND11_MODULE(_rt, m) {
       .def("finish", &Scheduler::finish)
       .def("append_tokens", &Scheduler::append_tokens)
       .def("schedule", &Scheduler::schedule, py::call_guard<py::gil_scoped_release>())
+      .def("extend", &Scheduler::extend, py::arg("id"), py::arg("tokens"))
+      .def("schedule_exact", &Scheduler::schedule_exact, py::arg("ids"), py::arg("counts"))
       .def("reserve_decode",
            [](Scheduler& s, const std::vector<int64_t>& ids, int steps) -> py::object {
              std::vector<int32_t> bt;

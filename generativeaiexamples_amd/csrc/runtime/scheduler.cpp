@@ -109,10 +109,6 @@ StepBatch Scheduler::schedule() {
     preempt(*seqs_[running_.back()]);
   }
 
-  struct Chunk {
-    Sequence* s;
-    int start, n;
-  };
   std::vector<Chunk> prefills;
   std::vector<Sequence*> decodes;
 
@@ -166,7 +162,57 @@ StepBatch Scheduler::schedule() {
     budget -= n;
   }
 
-  // ---- 4. flatten
+  flatten(prefills, decodes, b);
+  return b;
+}
+
+void Scheduler::extend(int64_t id, const std::vector<int>& toks) {
+  auto it = seqs_.find(id);
+  if (it == seqs_.end()) throw std::runtime_error("Scheduler.extend: unknown sequence");
+  Sequence& s = *it->second;
+  if ((int)(s.tokens.size() + toks.size()) > max_model_len_)
+    throw std::runtime_error("Scheduler.extend: sequence exceeds max_model_len");
+  s.tokens.insert(s.tokens.end(), toks.begin(), toks.end());
+  s.prompt_len = (int)s.tokens.size();
+}
+
+StepBatch Scheduler::schedule_exact(const std::vector<int64_t>& ids, const std::vector<int>& counts) {
+  if (ids.size() != counts.size()) throw std::runtime_error("schedule_exact: size mismatch");
+  int need = 0, admitted = 0;
+  for (size_t i = 0; i < ids.size(); ++i) {
+    auto it = seqs_.find(ids[i]);
+    if (it == seqs_.end()) throw std::runtime_error("schedule_exact: unknown sequence");
+    const Sequence& s = *it->second;
+    if (counts[i] < 1 || s.num_computed + counts[i] > (int)s.tokens.size())
+      throw std::runtime_error("schedule_exact: a sequence has fewer uncomputed tokens than asked for");
+    for (size_t j = 0; j < i; ++j)
+      if (ids[j] == ids[i]) throw std::runtime_error("schedule_exact: a sequence is named twice");
+    need += std::max(0, (s.num_computed + counts[i] + kBlockSize - 1) / kBlockSize - (int)s.blocks.size());
+    if (std::find(running_.begin(), running_.end(), ids[i]) == running_.end()) ++admitted;
+  }
+  if (!bm_.can_allocate(need)) throw std::runtime_error("schedule_exact: out of KV pages");
+  if ((int)running_.size() + admitted > max_num_seqs_) throw std::runtime_error("schedule_exact: too many sequences");
+  StepBatch b;
+  std::vector<Chunk> prefills;
+  std::vector<Sequence*> decodes;
+  for (size_t i = 0; i < ids.size(); ++i) {
+    Sequence& s = *seqs_[ids[i]];
+    auto w = std::find(waiting_.begin(), waiting_.end(), s.id);
+    if (w != waiting_.end()) {
+      waiting_.erase(w);
+      running_.push_back(s.id);
+    }
+    ensure_blocks(s, s.num_computed + counts[i]);
+    if (counts[i] == 1)
+      decodes.push_back(&s);
+    else
+      prefills.push_back({&s, s.num_computed, counts[i]});
+  }
+  flatten(prefills, decodes, b);
+  return b;
+}
+
+void Scheduler::flatten(std::vector<Chunk>& prefills, std::vector<Sequence*>& decodes, StepBatch& b) {
   int maxb = 0;
   for (auto& c : prefills) maxb = std::max(maxb, (int)c.s->blocks.size());
   for (auto* s : decodes) maxb = std::max(maxb, (int)s->blocks.size());
@@ -203,7 +249,6 @@ StepBatch Scheduler::schedule() {
     s.num_computed = pos + 1;
     commit_full_blocks(s);
   }
-  return b;
 }
 
 bool Scheduler::reserve_decode(const std::vector<int64_t>& ids, int steps, std::vector<int32_t>& block_tables,

@@ -66,6 +66,14 @@ class Scheduler {
 
   StepBatch schedule();
 
+  // Externally planned steps (replaying a recorded schedule, teacher-forced scoring): extend() appends tokens that
+  // the caller supplies to a sequence's prompt, and schedule_exact() builds the step that runs exactly counts[i] of
+  // the not yet computed tokens of ids[i] -- a single token as a decode row, more as a prefill portion, as schedule()
+  // classifies them -- admitting waiting sequences without a prefix-cache lookup. No preemption: it throws (and
+  // allocates nothing) when the KV pages do not suffice.
+  void extend(int64_t id, const std::vector<int>& toks);
+  StepBatch schedule_exact(const std::vector<int64_t>& ids, const std::vector<int>& counts);
+
   // Multi-step decode. After schedule() returned a pure-decode batch for `ids`, reserve KV pages so
   // each of them can run `steps` tokens (positions num_computed-1 .. num_computed+steps-2) with no
   // further scheduling; fills the [ids.size(), max_blocks] block tables. All-or-nothing: returns
@@ -93,6 +101,11 @@ class Scheduler {
   int num_generated(int64_t id) const;
 
  private:
+  struct Chunk {
+    Sequence* s;
+    int start, n;
+  };
+  void flatten(std::vector<Chunk>& prefills, std::vector<Sequence*>& decodes, StepBatch& b);
   bool ensure_blocks(Sequence& s, int upto_tokens);
   void release(Sequence& s);
   void commit_full_blocks(Sequence& s);

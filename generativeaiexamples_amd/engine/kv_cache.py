@@ -31,13 +31,25 @@ class KVCache:
     the attention kernels dequantise while loading - half the HBM bytes per cached token, twice the tokens."""
 
     def __init__(self, num_layers: int, num_blocks: int, num_kv_heads: int, head_dim: int, device,
-                 dtype=torch.bfloat16, k_scale: float = 1.0, v_scale: float = 1.0):
+                 dtype=torch.bfloat16, k_scale: float = 1.0, v_scale: float = 1.0, layout=None):
+        """``layout``: one (kv heads, key size, value size) per cache layer, for models whose attention layers differ
+        in head geometry or whose keys and values differ in size (each layer then has its own allocation, in the same
+        K [blocks, heads, 16, dk] / V^T [blocks, heads, dv, 16] page layout and with the same block ids)."""
+        if layout is not None:
+            num_layers = len(layout)
         self.num_layers, self.num_blocks = num_layers, num_blocks
         self.dtype = dtype
         fp8 = dtype == FP8
         self.k_scales = [float(k_scale) if fp8 else 1.0] * num_layers
         self.v_scales = [float(v_scale) if fp8 else 1.0] * num_layers
         self.hkv, self.hd = num_kv_heads, head_dim
+        self.layout = layout
+        if layout is not None:
+            # zero-filled for the same reason as below
+            self.k = [torch.zeros(num_blocks, g, BLOCK, dk, dtype=dtype, device=device) for g, dk, _ in layout]
+            self.v = [torch.zeros(num_blocks, g, dv, BLOCK, dtype=dtype, device=device) for g, _, dv in layout]
+            self.storage = None
+            return
         per = num_blocks * num_kv_heads * BLOCK * head_dim
         # zero-filled: masked tail slots of a page are read (and multiplied by p=0) by the kernels
         self.storage = torch.zeros(num_layers, 2, per, dtype=dtype, device=device)
@@ -51,6 +63,10 @@ class KVCache:
         return self.k_scales[i], self.v_scales[i]
 
     @staticmethod
+    def layout_bytes_per_block(layout, dtype=torch.bfloat16) -> int:
+        return sum(g * BLOCK * (dk + dv) for g, dk, dv in layout) * torch.finfo(dtype).bits // 8
+
+    @staticmethod
     def bytes_per_block(num_layers, num_kv_heads, head_dim, dtype=torch.bfloat16) -> int:
         return num_layers * 2 * num_kv_heads * BLOCK * head_dim * torch.finfo(dtype).bits // 8
 
@@ -60,4 +76,6 @@ class KVCache:
 
     @property
     def nbytes(self) -> int:
+        if self.storage is None:
+            return sum(t.numel() * t.element_size() for t in self.k + self.v)
         return self.storage.numel() * self.storage.element_size()

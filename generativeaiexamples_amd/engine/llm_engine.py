@@ -169,6 +169,11 @@ class LLMEngine:
             cfg.use_graphs = False  # host (gloo) collectives, e.g. a one-GPU TP rehearsal, are not capturable
         if self.tp_size > 1 and hasattr(model, "register_request"):
             raise NotImplementedError(f"{mc.name}: per-request model state is not replicated to TP followers")
+        if getattr(model, "has_recurrent_state", False):
+            cfg.prefix_cache = False  # cached prefix pages carry no recurrent state to resume from
+        self.window_attn = getattr(model, "attention_backend", "flash") == "window"
+        if hasattr(model, "set_state_slots"):  # one recurrent-state slot per sequence the scheduler may run
+            model.set_state_slots(cfg.max_num_seqs)
         self.kv_dtype = cache_dtype(cfg.kv_cache_dtype, model.dtype)
         if self.kv_dtype == torch.float8_e4m3fn and not getattr(model, "supports_fp8_kv", False):
             raise ValueError(f"{mc.name}: the fp8 KV cache is not supported by this model's attention path")
@@ -182,12 +187,13 @@ class LLMEngine:
         # one extra block, never handed out, is the scratch page of padded graph rows
         # models with non-KV layers (cross-attention) report how many layers own a paged KV cache
         self.kv = KVCache(self._kv_layers(), nb + 1, model.hkv, mc.head_dim, self.device, self.kv_dtype,
-                          k_scale=cfg.kv_scale, v_scale=cfg.kv_scale)
+                          k_scale=cfg.kv_scale, v_scale=cfg.kv_scale,
+                          layout=model.kv_layout() if hasattr(model, "kv_layout") else None)
         self.pad_block = nb
         self.sched = _rt().Scheduler(nb, cfg.max_num_seqs, cfg.max_batched_tokens, cfg.max_model_len,
                                      cfg.prefix_cache, cfg.prefill_chunk)
         self.decode_ws = None
-        if self.device.type == "cuda":
+        if self.device.type == "cuda" and not self.window_attn:
             self.decode_ws = ops.DecodeWorkspace(max(cfg.max_num_seqs, max(cfg.graph_batch_sizes)), model.hq,
                                                  mc.head_dim, max(cfg.max_model_len,
                                                                   getattr(model, "max_cross_tokens", 0)),
@@ -257,7 +263,11 @@ class LLMEngine:
             nbytes = int(free * frac)
         else:
             nbytes = 256 << 20
-        nb = KVCache.blocks_for_memory(nbytes, self._kv_layers(), self.model.hkv, mc.head_dim, self.kv_dtype)
+        if hasattr(self.model, "kv_layout"):  # per-layer head geometry
+            per = max(1, KVCache.layout_bytes_per_block(self.model.kv_layout(), self.kv_dtype))
+            nb = min(max(16, int(nbytes // per)), self.cfg.max_num_seqs * self.max_blocks_per_seq)
+        else:
+            nb = KVCache.blocks_for_memory(nbytes, self._kv_layers(), self.model.hkv, mc.head_dim, self.kv_dtype)
         return max(nb, 2 * self.max_blocks_per_seq)
 
     # ------------------------------------------------------------------ requests
@@ -383,22 +393,26 @@ class LLMEngine:
     # A step is planned on the TP leader (scheduler decisions, sampling parameters, KV pages) and executed
     # from the plan on every rank: the plan is a dict of numpy arrays and plain values, published unchanged
     # to the follower ranks (parallel/step_channel.py) when the model is tensor-parallel.
-    def _plan_eager(self, b) -> dict:
+    def _plan_eager(self, b, rows=None) -> dict:
+        """rows: the flat token rows whose logits the step returns (default: the last row of every prompt that
+        completes in this step, then every decode row)."""
         P = b.num_prefill_tokens
         samples = b.prefill_samples
         cu = b.cu_q
-        rows = []
-        for i, sid in enumerate(b.prefill_seq_ids):
-            if samples[i]:
-                rows.append(int(cu[i + 1]) - 1)
         nd = len(b.decode_seq_ids)
-        rows += range(P, P + nd)
+        if rows is None:
+            rows = []
+            for i, sid in enumerate(b.prefill_seq_ids):
+                if samples[i]:
+                    rows.append(int(cu[i + 1]) - 1)
+            rows += range(P, P + nd)
         arrs = [b.token_ids, b.positions, b.slots, cu, b.prefill_ctx, b.prefill_block_tables, b.decode_ctx,
                 b.decode_block_tables, np.asarray(rows, dtype=np.int32)]
-        if P > 0:
+        if P > 0 and not self.window_attn:
             rpt = ops.prefill_rows_per_tile(self.model.hq, self.model.hkv, self.model.cfg.head_dim)
             arrs.append(ops.prefill_tile_list(b.prefill_qlen, rpt, b.prefill_ctx))
         plan = dict(op="eager", P=int(P), arr=arrs, qlen=[int(x) for x in b.prefill_qlen],
+                    dctx=[int(x) for x in b.decode_ctx],
                     pctx=[int(x) for x in b.prefill_ctx], max_dctx=int(b.decode_ctx.max()) if nd else 0,
                     seq_ids=[int(x) for x in b.prefill_seq_ids] + [int(x) for x in b.decode_seq_ids],
                     pseq=[int(x) for x, smp in zip(b.prefill_seq_ids, samples) if smp])
@@ -416,10 +430,12 @@ class LLMEngine:
             fb.cu_q, fb.prefill_ctx, fb.prefill_block_tables = dev[3], dev[4], dev[5]
             fb.prefill_qlen = list(plan["qlen"])
             fb.prefill_ctx_host = list(plan["pctx"])
-            fb.prefill_tiles = dev[9].reshape(-1)
+            if not self.window_attn:
+                fb.prefill_tiles = dev[9].reshape(-1)
         if plan["max_dctx"]:
             fb.decode_ctx, fb.decode_block_tables = dev[6], dev[7]
             fb.max_decode_ctx = plan["max_dctx"]
+            fb.decode_ctx_host = list(plan.get("dctx") or [])
         fb.sample_rows = dev[8].long()
         fb.seq_ids = list(plan["seq_ids"])
         if plan.get("lora") is not None:
@@ -1060,6 +1076,69 @@ class LLMEngine:
         if cont_ids and not defer_append:
             self.sched.append_tokens(cont_ids, cont_toks)
         return outs
+
+    # ------------------------------------------------------------------ externally planned steps
+    @torch.inference_mode()
+    def replay_step(self, entries, end=()) -> Optional[torch.Tensor]:
+        """One step of an externally planned schedule (replaying a recorded trace, teacher-forced scoring): nothing is
+        sampled. ``entries``: (request id, the request's next token ids, offsets among them whose logits are wanted);
+        a request is admitted at its first entry and may sit out a step. ``end``: request ids finished after the step
+        (their KV pages and state slot return to the pools). All entries run as ONE batch through the engine's own
+        plan / staging / forward path - prompt portions next to single tokens; a step of single tokens only replays
+        the captured decode graph, as generation does. Returns fp32 logits [wanted, vocab] on the host, in the order
+        of the entries and their offsets (None when nothing is wanted)."""
+        with self.lock:
+            ids, counts = [], []
+            for rid, toks, _want in entries:
+                toks = [int(t) for t in toks]
+                req = self.by_rid.get(rid)
+                if req is None:
+                    sid = next(self._ids)
+                    req = Request(rid, toks, SamplingParams(max_tokens=0), sid, IncrementalDetokenizer(self.tok, ()))
+                    self.requests[sid] = self.by_rid[rid] = req
+                    self.sched.add(sid, toks, 0)
+                else:
+                    req.prompt_ids += toks
+                    self.sched.extend(req.seq_id, toks)
+                ids.append(req.seq_id)
+                counts.append(len(toks))
+            out = None
+            if ids:
+                b = self.sched.schedule_exact(ids, counts)
+                P, nd = b.num_prefill_tokens, len(b.decode_seq_ids)
+                cu = b.cu_q
+                start = {int(sid): int(cu[i]) for i, sid in enumerate(b.prefill_seq_ids)}
+                start.update({int(sid): P + j for j, sid in enumerate(b.decode_seq_ids)})
+                rows = [start[sid] + int(k) for sid, (_r, _t, want) in zip(ids, entries) for k in want]
+                self.step_count += 1
+                self.stats["steps"] += 1
+                self.stats["prefill_tokens"] += P
+                self.stats["decode_tokens"] += nd
+                st = self._bank()
+                if P == 0 and self.device.type == "cuda" and self.cfg.use_graphs and self._graph_bucket(nd) is not None:
+                    plan = dict(op="graph", n=nd, arr=[b.token_ids, b.positions, b.slots, b.decode_ctx,
+                                                        b.decode_block_tables],
+                                seq_ids=[int(x) for x in b.decode_seq_ids])
+                    logits = self._run_graph(plan)
+                    if rows:
+                        out = logits.index_select(0, self._to_device([np.asarray(rows, np.int32)])[0].long())
+                else:
+                    fb = self._batch_from_plan(self._plan_eager(b, rows=rows))
+                    logits = self.model.forward(fb, self.kv, self.decode_ws)
+                    if rows:
+                        out = logits
+                if out is not None:
+                    out = out.float().cpu()
+                st.fence()
+                self._step_done()
+            for rid in end:
+                req = self.by_rid.pop(rid, None)
+                if req is not None:
+                    self.sched.finish(req.seq_id)
+                    self.requests.pop(req.seq_id, None)
+                    self._release(req.seq_id)
+                    req.finished, req.finish_reason = True, "stop"
+            return out
 
     # ------------------------------------------------------------------ offline API
     def generate(self, prompts: List[List[int]], params: SamplingParams | List[SamplingParams] | None = None

@@ -29,6 +29,7 @@ class ForwardBatch:
     decode_ctx: Optional[torch.Tensor] = None      # [Dn] int32
     decode_block_tables: Optional[torch.Tensor] = None  # [Dn, maxb] int32
     max_decode_ctx: int = 0
+    decode_ctx_host: List[int] = field(default_factory=list)   # host copy of decode_ctx (state-slot models)
     # rows of the flat token dim whose logits are needed (in output order)
     sample_rows: Optional[torch.Tensor] = None     # [S] int64
     # host-side sequence ids of the rows (prefill sequences, then decode sequences) and model-specific

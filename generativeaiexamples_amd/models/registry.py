@@ -15,6 +15,7 @@ from .llama import LlamaConfig, LlamaModel
 from .mixtral import MixtralConfig, MixtralModel
 from .mllama import MllamaConfig, MllamaModel
 from .opt import OPTConfig, OPTModel
+from .pinavik import PinavikConfig, PinavikModel
 from .qwen3_next import Qwen3NextConfig, Qwen3NextModel
 
 LLM_PRESETS = {
@@ -36,6 +37,9 @@ LLM_PRESETS = {
     "qwen3-next-80b-a3b-thinking": ("qwen/qwen3-next-80b-a3b-thinking",
                                     lambda: Qwen3NextConfig.qwen3_next_80b_a3b(name="qwen/qwen3-next-80b-a3b-thinking")),
     "tiny-qwen3-next": ("tiny-qwen3-next", lambda: Qwen3NextConfig.tiny()),
+    # hybrid of windowed attention, WKV and channel-decay delta-rule layers with a looped block (fp32 residual / state)
+    "tiny-pinavik": ("tiny-pinavik", lambda: PinavikConfig.tiny()),
+    "pinavik-1b": ("pinavik-1b", lambda: PinavikConfig.sized(2048, 18, 5632, 16, 128)),
     "opt-125m": ("facebook/opt-125m", lambda: OPTConfig.opt_125m()),
     "mixtral-8x7b": ("mistralai/mixtral-8x7b-instruct-v0.1", lambda: MixtralConfig.mixtral_8x7b()),
     "tiny-moe": ("tiny-moe", lambda: MixtralConfig.tiny_moe()),
@@ -71,8 +75,11 @@ def build_llm(preset: str = "llama3-8b", weights: Optional[str] = None, device=N
     if _is_hf_dir(weights):
         import json
 
-        arch = json.load(open(os.path.join(weights, "config.json"))).get("model_type", "llama")
-        if arch == "opt":
+        hf = json.load(open(os.path.join(weights, "config.json")))
+        arch = hf.get("model_type") or str(hf.get("architecture", "llama")).lower()
+        if arch == "pinavik":
+            m = PinavikModel(PinavikConfig.from_json(weights), device=device, dtype=dtype or torch.bfloat16)
+        elif arch == "opt":
             m = OPTModel(OPTConfig.from_hf(weights), device=device)
         elif arch == "mixtral":
             m = MixtralModel(MixtralConfig.from_hf(weights), device=device)
@@ -102,6 +109,9 @@ def build_llm(preset: str = "llama3-8b", weights: Optional[str] = None, device=N
         vocab = cfg.vocab_size
     elif isinstance(cfg, Qwen3NextConfig):
         m = Qwen3NextModel(cfg, device=device).random_init(seed)
+        vocab = cfg.vocab_size
+    elif isinstance(cfg, PinavikConfig):
+        m = PinavikModel(cfg, device=device, dtype=dtype or torch.bfloat16).random_init(seed)
         vocab = cfg.vocab_size
     else:
         m = LlamaModel(cfg, device=device).random_init(seed)

@@ -114,6 +114,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
         return _into(out, ref.linear(x, w, bias, residual, act, out_dtype))
     K = x.shape[-1]
     N = w.shape[0]
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or K % 64 or N % 16:
+        return _vendor_linear(x, w, bias, residual, act, out_dtype, out)
     lead = x.shape[:-1]
     M = x.numel() // K
     out_dtype = out_dtype or x.dtype
@@ -148,6 +150,23 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
         out = torch.empty(*lead, ncol, dtype=out_dtype, device=x.device)
     _native_gemm(x2, w, out, bias, residual, epi)
     return out
+
+
+def _vendor_linear(x, w, bias, residual, act, out_dtype, out):
+    """rocBLAS / hipBLASLt product for what the hand-written MFMA kernels do not take: fp32 operands (true fp32: no
+    reduced-precision matrix mode is switched on) and bf16 shapes off their tile grid (K % 64, N % 16). fp32 output
+    from bf16 operands is computed from the upcast operands."""
+    if act is not None:
+        raise ValueError(f"linear: activation {act!r} needs bf16 operands with K % 64 == 0 and N % 16 == 0")
+    wn = natural_weight(w)
+    od = out_dtype or x.dtype
+    if x.dtype == torch.float32 or od == torch.float32:
+        y = torch.nn.functional.linear(x.float(), wn.float(), None if bias is None else bias.float())
+    else:
+        y = torch.nn.functional.linear(x, wn.to(x.dtype), None if bias is None else bias.to(x.dtype))
+    if residual is not None:
+        y = y + residual
+    return _into(out, y.to(od))
 
 
 _SPLITK = os.environ.get("GAI_SPLITK", "1") == "1"
@@ -1012,4 +1031,131 @@ def vit_embed(patches: torch.Tensor, cls: torch.Tensor, pos: torch.Tensor, B: in
     NP = patches.numel() // (B * D)
     out = torch.empty(B * (NP + 1), D, dtype=torch.bfloat16, device=patches.device)
     native().vit_embed(patches, cls, pos, out, B)
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
+# sequence mixers with a 32-bit residual / state (hybrid decoders)
+#
+# A step's rows are S sequences [cu[s], cu[s+1]) (prompt portions and single decoded tokens alike) with per-sequence
+# pool slots; cu / slots / ctx / block tables are int32 device vectors, so a decode step is graph-capturable.
+# Activations are bf16 or fp32; residual, statistics, scores, decays and states are fp32.
+# ---------------------------------------------------------------------------------------------
+def add_rmsnorm_f32(res: torch.Tensor, delta: Optional[torch.Tensor] = None, mult: float = 1.0,
+                    w: Optional[torch.Tensor] = None, eps: float = 1e-6, out_dtype=None):
+    """fp32 residual ``res`` (in place) += mult * delta, then (out_dtype given) rmsnorm(res) * w -- or res itself
+    when w is None -- in out_dtype. One pass: the residual add of one block and the norm of the next."""
+    if not res.is_cuda:
+        return ref.add_rmsnorm_f32(res, delta, mult, w, eps, out_dtype)
+    out = torch.empty(res.shape, dtype=out_dtype, device=res.device) if out_dtype is not None else None
+    native().add_rmsnorm_f32(res, delta, float(mult), w, out, float(eps))
+    return out
+
+
+def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """a N(z) + b N(z^2) + c N(z^3) + e over the last dim, N = division by the root mean square; coef = (a, b, c, e)."""
+    if not z.is_cuda:
+        return ref.poly_norm(z, coef, eps)
+    y = torch.empty_like(z)
+    native().poly_norm(z, coef, float(eps), y)
+    return y
+
+
+def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, nw: torch.Tensor, act: str, eps: float, out_dtype):
+    """Per-head RMS norm of fp32 o [T, H, DV], times nw ([H * DV] or shared [DV]), times silu / sigmoid of gate."""
+    a = {"silu": 0, "sigmoid": 1}[act]
+    if not o.is_cuda:
+        return ref.head_norm_gate(o, gate, nw, a, eps, out_dtype)
+    T, H, DV = o.shape
+    y = torch.empty(T, H * DV, dtype=out_dtype, device=o.device)
+    native().head_norm_gate(o, gate, nw, a, float(eps), y)
+    return y
+
+
+def embed_scale_f32(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+    if not table.is_cuda:
+        return ref.embed_scale_f32(ids, table, scale)
+    out = torch.empty(ids.numel(), table.shape[1], dtype=torch.float32, device=table.device)
+    native().embed_scale_f32(ids, table, float(scale), out)
+    return out
+
+
+def qknorm_kv_write(q, k, v, wq, wk, slots, k_cache, v_cache, H: int, G: int, DK: int, DV: int, eps: float):
+    """RMS norm over the whole q row and the whole k row (weights wq / wk), k and v into their cache slots;
+    returns the normalised q [T, H * DK]. q / k / v may be column slices of one projection output."""
+    if not q.is_cuda:
+        return ref.qknorm_kv_write(q, k, v, wq, wk, slots, k_cache, v_cache, H, G, DK, DV, eps)
+    q_out = torch.empty(q.shape[0], H * DK, dtype=q.dtype, device=q.device)
+    native().qknorm_kv_write(q, k, v, wq, wk, slots, q_out, k_cache, v_cache, H, G, DK, DV, float(eps))
+    return q_out
+
+
+def window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H: int, G: int, DK: int, DV: int, scale: float,
+                     softcap: float = 0.0, window: int = 0, r1=None, r2=None, gate=None):
+    """Sliding-window paged attention, scores capped by softcap * tanh(s / softcap) and lowered by
+    r1_h ln(1 + r2_h distance); output [T, H * DV], times sigmoid(gate) when given."""
+    if not q.is_cuda:
+        return ref.window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H, G, DK, DV, scale, softcap, window,
+                                    r1, r2, gate)
+    out = torch.empty(q.shape[0], H * DV, dtype=q.dtype, device=q.device)
+    native().window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, out, H, G, DK, DV, float(scale),
+                              float(softcap or 0.0), int(window or 0), r1, r2, gate)
+    return out
+
+
+def token_shift_mix(h, mu, shift_state, cu, slots):
+    """[NM, T, D]: h + (previous row - h) * mu_n; the row before a sequence's first comes from shift_state[slot]."""
+    if not h.is_cuda:
+        return ref.token_shift_mix(h, mu, shift_state, cu, slots)
+    out = torch.empty(mu.shape[0], *h.shape, dtype=h.dtype, device=h.device)
+    native().token_shift_mix(h, mu, shift_state, cu, slots, out)
+    return out
+
+
+def state_tail_write(x, state, cu, slots) -> None:
+    """state[slot] ([rows, C] fp32) <- the last rows of (state[slot] | x[cu[s]:cu[s+1]])."""
+    if not x.is_cuda:
+        return ref.state_tail_write(x, state, cu, slots)
+    native().state_tail_write(x, state, cu, slots)
+
+
+def conv_silu(x, w, state, cu, slots):
+    """Causal depthwise conv over time (w [C, taps], last tap = current row) + SiLU -> fp32 [T, C]."""
+    if not x.is_cuda:
+        return ref.conv_silu(x, w, state, cu, slots)
+    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    native().conv_silu(x, w, state, cu, slots, y)
+    return y
+
+
+def wkv_scan(r, k, v, wpre, w0, u, state, cu, slots):
+    """WKV recurrence with bonus u and decay exp(-exp(wpre + w0)); state [slots, H, D, D] in place -> fp32 [T, H, D]."""
+    if not r.is_cuda:
+        return ref.wkv_scan(r, k, v, wpre, w0, u, state, cu, slots)
+    H, D = state.shape[1], state.shape[2]
+    out = torch.empty(r.shape[0], H, D, dtype=torch.float32, device=r.device)
+    native().wkv_scan(r, k, v, wpre, w0, u, state, cu, slots, out)
+    return out
+
+
+def delta_prep(qkv, a, b, A_log, dt_bias, H: int, G: int, DK: int):
+    """Delta-rule inputs: unit q (x DK^-1/2) / k [T, G, DK], decay [T, H, DK], beta [T, H] (all fp32)."""
+    if not qkv.is_cuda:
+        return ref.delta_prep(qkv, a, b, A_log, dt_bias, H, G, DK)
+    T, dev = qkv.shape[0], qkv.device
+    qn = torch.empty(T, G, DK, dtype=torch.float32, device=dev)
+    kn = torch.empty_like(qn)
+    decay = torch.empty(T, H, DK, dtype=torch.float32, device=dev)
+    beta = torch.empty(T, H, dtype=torch.float32, device=dev)
+    native().delta_prep(qkv, a, b, A_log, dt_bias, qn, kn, decay, beta, H, G, DK)
+    return qn, kn, decay, beta
+
+
+def delta_scan(q, k, v, decay, beta, state, cu, slots, G: int):
+    """Gated delta rule with a decay per key channel; state [slots, H, DK, DV] in place -> fp32 [T, H, DV]."""
+    if not v.is_cuda:
+        return ref.delta_scan(q, k, v, decay, beta, state, cu, slots, G)
+    H, DV = state.shape[1], state.shape[3]
+    out = torch.empty(v.shape[0], H, DV, dtype=torch.float32, device=v.device)
+    native().delta_scan(q, k, v, decay, beta, state, cu, slots, out, G)
     return out

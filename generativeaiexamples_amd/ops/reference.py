@@ -441,3 +441,158 @@ def vit_embed(patches: torch.Tensor, cls: torch.Tensor, pos: torch.Tensor, B: in
     p = patches.float().reshape(B, -1, D)
     x = torch.cat([cls.float().view(1, 1, D).expand(B, 1, D), p], 1) + pos.float()[: p.shape[1] + 1]
     return x.reshape(-1, D).to(torch.bfloat16)
+
+
+# ---------------------------------------------------------------------------------------------
+# sequence mixers with a 32-bit residual / state (window attention, WKV, channel-decay delta rule)
+# ---------------------------------------------------------------------------------------------
+def _seqs(cu, slots):
+    c = [int(x) for x in cu.tolist()]
+    return [(c[i], c[i + 1], int(s)) for i, s in enumerate(slots.tolist())]
+
+
+def add_rmsnorm_f32(res, delta, mult, w, eps, out_dtype):
+    """res (fp32, in place) += mult * delta; returns rms-normalised res * w (w None: res itself) as out_dtype."""
+    if delta is not None:
+        res.add_(delta.float(), alpha=float(mult))
+    if out_dtype is None:
+        return None
+    if w is None:
+        return res.to(out_dtype)
+    return (res * torch.rsqrt(res.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def poly_norm(z, coef, eps):
+    x = z.float()
+    n = lambda t: t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps)  # noqa: E731
+    a, b, c, e = [float(v) for v in coef.tolist()]
+    return (a * n(x) + b * n(x * x) + c * n(x * x * x) + e).to(z.dtype)
+
+
+def head_norm_gate(o, gate, nw, act, eps, out_dtype):
+    T, H, DV = o.shape
+    y = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps)
+    y = y * (nw.float().view(H, DV) if nw.numel() == H * DV else nw.float())
+    g = gate.float().reshape(T, H, DV)
+    y = y * (F.silu(g) if act == 0 else torch.sigmoid(g))
+    return y.reshape(T, H * DV).to(out_dtype)
+
+
+def embed_scale_f32(ids, table, scale):
+    return table[ids.long().clamp(0, table.shape[0] - 1)].float() * float(scale)
+
+
+def qknorm_kv_write(q, k, v, wq, wk, slots, k_cache, v_cache, H, G, DK, DV, eps):
+    T = q.shape[0]
+    n = lambda t, w: t.float() * torch.rsqrt(t.float().pow(2).mean(-1, keepdim=True) + eps) * w.float()  # noqa: E731
+    qn = n(q, wq).to(q.dtype)
+    kn = n(k, wk).to(k_cache.dtype).view(T, G, DK)
+    s = slots[:T].long()
+    k_cache[s // BLOCK, :, s % BLOCK] = kn
+    v_cache[s // BLOCK, :, :, s % BLOCK] = v.reshape(T, G, DV).to(v_cache.dtype)
+    return qn
+
+
+def window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H, G, DK, DV, scale, softcap, window, r1, r2, gate):
+    T = q.numel() // (H * DK)
+    q3 = q.float().view(T, H, DK)
+    out = torch.zeros(T, H, DV)
+    cu = [int(x) for x in cu_q.tolist()]
+    for s, n in enumerate(ctx.tolist()):
+        b, e = cu[s], cu[s + 1]
+        if e <= b:
+            continue
+        n = int(n)
+        pages = block_tables[s, : (n + BLOCK - 1) // BLOCK].long()
+        K = k_cache[pages].float().permute(1, 0, 2, 3).reshape(G, -1, DK)[:, :n]          # [G, n, DK]
+        V = v_cache[pages].float().permute(1, 0, 3, 2).reshape(G, -1, DV)[:, :n]          # [G, n, DV]
+        pos = torch.arange(n - (e - b), n)
+        dist = pos[:, None] - torch.arange(n)[None, :]
+        vis = (dist >= 0) & ((dist < window) if window > 0 else True)
+        for h in range(H):
+            sc = (q3[b:e, h] @ K[h // (H // G)].t()) * scale
+            if softcap > 0:
+                sc = softcap * torch.tanh(sc / softcap)
+            if r1 is not None:
+                sc = sc - float(r1[h]) * torch.log1p(float(r2[h]) * dist.clamp(min=0).float())
+            sc = sc.masked_fill(~vis, float("-inf"))
+            out[b:e, h] = torch.softmax(sc, -1) @ V[h // (H // G)]
+    out = out.reshape(T, H * DV)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float())
+    return out.to(q.dtype)
+
+
+def token_shift_mix(h, mu, shift_state, cu, slots):
+    x = h.float()
+    prev = torch.empty_like(x)
+    prev[1:] = x[:-1]
+    for b, e, s in _seqs(cu, slots):
+        if e > b:
+            prev[b] = shift_state[s]
+    return (x[None] + (prev - x)[None] * mu.float()[:, None]).to(h.dtype)
+
+
+def state_tail_write(x, state, cu, slots):
+    NR = state.shape[1]
+    for b, e, s in _seqs(cu, slots):
+        if e > b:
+            state[s] = torch.cat([state[s], x[b:e].float()])[-NR:]
+
+
+def conv_silu(x, w, state, cu, slots):
+    K = w.shape[1]
+    y = torch.empty(x.shape, dtype=torch.float32)
+    for b, e, s in _seqs(cu, slots):
+        if e > b:
+            xs = torch.cat([state[s], x[b:e].float()])
+            y[b:e] = (xs.unfold(0, K, 1) * w.float()).sum(-1)
+    return F.silu(y)
+
+
+def wkv_scan(r, k, v, wpre, w0, u, state, cu, slots):
+    H, D = state.shape[1], state.shape[2]
+    T = r.shape[0]
+    r3, k3, v3 = (t.float().reshape(T, H, D) for t in (r, k, v))
+    w = torch.exp(-torch.exp(wpre.float().reshape(T, H, D) + w0.float().reshape(H, D)))
+    uu = u.float().reshape(H, D)
+    out = torch.empty(T, H, D)
+    for b, e, s in _seqs(cu, slots):
+        S = state[s]
+        for t in range(b, e):
+            kv = k3[t][:, :, None] * v3[t][:, None, :]
+            out[t] = torch.einsum("hkv,hk->hv", S + uu[:, :, None] * kv, r3[t])
+            S = w[t][:, :, None] * S + kv
+        if e > b:
+            state[s] = S
+    return out
+
+
+def delta_prep(qkv, a, b, A_log, dt_bias, H, G, DK):
+    T = qkv.shape[0]
+    l2 = lambda t: t * torch.rsqrt(t.pow(2).sum(-1, keepdim=True) + 1e-6)  # noqa: E731
+    qn = l2(qkv[:, : G * DK].float().reshape(T, G, DK)) * DK ** -0.5
+    kn = l2(qkv[:, G * DK: 2 * G * DK].float().reshape(T, G, DK))
+    sp = F.softplus(a.float() + dt_bias.float().reshape(1, -1)).reshape(T, H, DK)
+    decay = torch.exp(-torch.exp(A_log.float())[None, :, None] * sp)
+    return qn, kn, decay, torch.sigmoid(b.float())
+
+
+def delta_scan(q, k, v, decay, beta, state, cu, slots, G):
+    H, DK, DV = state.shape[1:]
+    T = v.shape[0]
+    rep = H // G
+    q3 = q.reshape(T, G, DK).repeat_interleave(rep, 1)
+    k3 = k.reshape(T, G, DK).repeat_interleave(rep, 1)
+    v3 = v.float().reshape(T, H, DV)
+    out = torch.empty(T, H, DV)
+    for b, e, s in _seqs(cu, slots):
+        S = state[s]
+        for t in range(b, e):
+            S = decay[t][:, :, None] * S
+            u = beta[t][:, None] * (v3[t] - torch.einsum("hkv,hk->hv", S, k3[t]))
+            S = S + k3[t][:, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hkv,hk->hv", S, q3[t])
+        if e > b:
+            state[s] = S
+    return out
