@@ -140,9 +140,23 @@ def small_byte_tokenizer(vocab_size: int = 512) -> ByteTokenizer:
     return ByteTokenizer(vocab_size, 8, sp, bos="<s>", eos=("</s>", "<|eot_id|>"))
 
 
+class FoldedByteTokenizer(ByteTokenizer):
+    """For a checkpoint without tokenizer files whose vocabulary is smaller than a byte table: text bytes are folded
+    modulo the vocabulary (lossy). Such models are driven by token ids; this keeps the text entry points total."""
+
+    def __init__(self, vocab_size: int):
+        super().__init__(0, 0)
+        self.vocab_size = vocab_size
+
+    def _bytes_ids(self, piece: str) -> List[int]:
+        return [b % self.vocab_size for b in piece.encode("utf-8")]
+
+
 def load_tokenizer(path: Optional[str], family: str = "llama3", vocab_size: Optional[int] = None) -> Tokenizer:
     if path and (os.path.isfile(path) or os.path.isfile(os.path.join(path, "tokenizer.json"))):
         return HFTokenizer(path)
+    if vocab_size is not None and 0 < vocab_size < 264:
+        return FoldedByteTokenizer(vocab_size)
     if family == "bert":
         return bert_byte_tokenizer(vocab_size or 30522)
     if family == "llama3" and (vocab_size is None or vocab_size >= 128256):

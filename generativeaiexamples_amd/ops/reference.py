@@ -535,6 +535,8 @@ def token_shift_mix(h, mu, shift_state, cu, slots):
 
 def state_tail_write(x, state, cu, slots):
     NR = state.shape[1]
+    if NR == 0:
+        return
     for b, e, s in _seqs(cu, slots):
         if e > b:
             state[s] = torch.cat([state[s], x[b:e].float()])[-NR:]
