@@ -96,6 +96,8 @@ def parse():
     from generativeaiexamples_amd.benchmarks import CONFIGS, module
     for c in CONFIGS:
         module(c).add_args(ap)
+    from generativeaiexamples_amd.benchmarks import hybrid
+    hybrid.add_args(ap)
     return ap.parse_args()
 
 
@@ -202,6 +204,15 @@ def synthetic_question(q: int) -> str:
 
 def main():
     args = parse()
+    if args.hybrid:  # model-level prefill / decode throughput of the hybrid decoders (one GPU, own JSON line)
+        from generativeaiexamples_amd.benchmarks import hybrid
+
+        out = hybrid.run(args)
+        print(json.dumps(out), flush=True)
+        if args.json_out:
+            with open(args.json_out, "w") as f:
+                json.dump(out, f)
+        return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         from generativeaiexamples_amd.parallel.launch import spawn_ranks
 

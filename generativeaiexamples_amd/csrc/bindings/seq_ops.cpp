@@ -186,7 +186,7 @@ void wkv_scan(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& w
                   u.numel() == H * D && cu.numel() == S + 1 && out.numel() == (int64_t)T * H * D,
               "wkv_scan: decay / bonus / cu / out shapes");
   gai_wkv_scan(r.data_ptr(), k.data_ptr(), v.data_ptr(), ld, f32(wpre, "wpre"), f32(w0, "w0"), f32(u, "u"),
-               f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, f32w(out, "out"), H, D, dt, cur_stream());
+               f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, T, f32w(out, "out"), H, D, dt, cur_stream());
 }
 
 void delta_prep(const Tensor& qkv, const Tensor& a, const Tensor& b, const Tensor& A_log, const Tensor& dt_bias,
@@ -216,7 +216,7 @@ void delta_scan(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor&
                   beta.numel() == (int64_t)T * H && cu.numel() == S + 1 && out.numel() == (int64_t)T * H * DV,
               "delta_scan: q / k / decay / beta / cu / out shapes");
   gai_delta_scan(f32(q, "q"), f32(k, "k"), v.data_ptr<float>(), (int)v.stride(0), f32(decay, "decay"), f32(beta, "beta"),
-                 f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, f32w(out, "out"), H, G, DK, DV,
+                 f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, T, f32w(out, "out"), H, G, DK, DV,
                  cur_stream());
 }
 

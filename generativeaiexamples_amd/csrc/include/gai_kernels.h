@@ -224,11 +224,11 @@ void gai_state_tail_write(const void* x, int ldx, float* state, const int* cu, c
 void gai_conv_silu(const void* x, int ldx, const float* w, const float* state, const int* cu, const int* slots, int S,
                    float* y, int T, int C, int K, int dt, hipStream_t st);
 void gai_wkv_scan(const void* r, const void* k, const void* v, int ld, const float* wpre, const float* w0,
-                  const float* u, float* state, const int* cu, const int* slots, int S, float* out, int H, int D,
+                  const float* u, float* state, const int* cu, const int* slots, int S, int T, float* out, int H, int D,
                   int dt, hipStream_t st);
 void gai_delta_prep(const float* qkv, int ld, const void* a, int lda, const void* b, int ldb, const float* A_log,
                     const float* dt_bias, float* qn, float* kn, float* decay, float* beta, int T, int H, int G, int DK,
                     int dt, hipStream_t st);
 void gai_delta_scan(const float* q, const float* k, const float* v, int ldv, const float* decay, const float* beta,
-                    float* state, const int* cu, const int* slots, int S, float* out, int H, int G, int DK, int DV,
-                    hipStream_t st);
+                    float* state, const int* cu, const int* slots, int S, int T, float* out, int H, int G, int DK,
+                    int DV, hipStream_t st);

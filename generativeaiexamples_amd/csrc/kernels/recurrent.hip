@@ -255,6 +255,208 @@ __global__ __launch_bounds__(1024) void delta_scan_kernel(const float* __restric
     if (i < nrow) Sg[(size_t)i * DV] = col[i];
 }
 
+// ---- prompt portions: one wave64 per (head, sequence, block of state columns) -------------------------------------
+// The columns of S evolve independently of each other, so a long portion is spread over many waves per head instead
+// of one workgroup: lane (rg, jj) owns rows [rg R, rg R + R) of column jj (RGS row groups x 64 / RGS columns), the token
+// inputs of 8 tokens at a time are staged in LDS by the wave itself (coalesced loads, prefetched into registers one
+// round ahead), and the row-group reductions are lane shuffles: no workgroup barrier anywhere in the token loop. LDS
+// rows past DK stay zero, so the token loop has no row guard (branch-free: its LDS reads are issued in batches).
+constexpr int kTB = 8;
+
+template <int R>
+__device__ __forceinline__ int lds_row(int row) { return row + row / R; }  // row groups land in different banks
+
+template <int COLS>
+__device__ __forceinline__ float rowgroup_sum(float v) {
+#pragma unroll
+  for (int o = COLS; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+template <typename TA, int R, int RGS>
+__global__ __launch_bounds__(64) void wkv_scan_cols_kernel(const TA* __restrict__ r, const TA* __restrict__ k,
+                                                           const TA* __restrict__ v, int ld, const float* __restrict__ wpre,
+                                                           const float* __restrict__ w0, const float* __restrict__ u,
+                                                           float* __restrict__ state, const int* __restrict__ cu,
+                                                           const int* __restrict__ slots, float* __restrict__ out, int H,
+                                                           int D) {
+  constexpr int COLS = 64 / RGS, NP = kTB * RGS * R / 64, LD = RGS * R + RGS;
+  extern __shared__ float lds[];
+  const int h = blockIdx.x, s = blockIdx.y, cb = blockIdx.z, lane = threadIdx.x;
+  const int jj = lane % COLS, rg = lane / COLS, j = cb * COLS + jj;
+  const bool on = j < D;
+  const int row0 = rg * R, nrow = max(0, min(R, D - row0));
+  float* rs = lds;
+  float* ks = rs + kTB * LD;
+  float* ws = ks + kTB * LD;
+  float* vs = ws + kTB * LD;  // [kTB][COLS]
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;
+  for (int x = lane; x < 3 * kTB * LD; x += 64) lds[x] = 0.f;
+  float* Sg = state + (((size_t)slots[s] * H + h) * D + row0) * D + j;
+  float col[R], ur[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    col[i] = (on && i < nrow) ? Sg[(size_t)i * D] : 0.f;
+    ur[i] = i < nrow ? u[(size_t)h * D + row0 + i] : 0.f;
+  }
+  float pr[NP], pk[NP], pw[NP], pv[2];
+  auto fetch = [&](int tb) {
+    const int n = min(kTB, t1 - tb);
+#pragma unroll
+    for (int x = 0; x < NP; ++x) {
+      const int idx = x * 64 + lane, tt = idx / D, i = idx - tt * D;
+      if (tt < n) {
+        const size_t o = (size_t)(tb + tt) * ld + (size_t)h * D + i;
+        pr[x] = (float)r[o];
+        pk[x] = (float)k[o];
+        pw[x] = wpre[((size_t)(tb + tt) * H + h) * D + i] + w0[(size_t)h * D + i];
+      }
+    }
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+      const int idx = x * 64 + lane, tt = idx / COLS, c = cb * COLS + idx % COLS;
+      pv[x] = (tt < n && c < D) ? (float)v[(size_t)(tb + tt) * ld + (size_t)h * D + c] : 0.f;
+    }
+  };
+  fetch(t0);
+  for (int tb = t0; tb < t1; tb += kTB) {
+    const int n = min(kTB, t1 - tb);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int x = 0; x < NP; ++x) {
+      const int idx = x * 64 + lane, tt = idx / D, i = idx - tt * D;
+      if (tt < n) {
+        const int a = tt * LD + lds_row<R>(i);
+        rs[a] = pr[x];
+        ks[a] = pk[x];
+        ws[a] = expf(-expf(pw[x]));
+      }
+    }
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+      if (x * 64 + lane < kTB * COLS) vs[x * 64 + lane] = pv[x];
+    __builtin_amdgcn_wave_barrier();
+    if (tb + kTB < t1) fetch(tb + kTB);
+    for (int tt = 0; tt < n; ++tt) {
+      const float vj = vs[tt * COLS + jj];
+      const int a = tt * LD + row0 + rg;
+      float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < R; i += 2) {
+        const float kv0 = ks[a + i] * vj, kv1 = ks[a + i + 1] * vj;
+        acc0 = fmaf(rs[a + i], fmaf(ur[i], kv0, col[i]), acc0);
+        acc1 = fmaf(rs[a + i + 1], fmaf(ur[i + 1], kv1, col[i + 1]), acc1);
+        col[i] = fmaf(ws[a + i], col[i], kv0);
+        col[i + 1] = fmaf(ws[a + i + 1], col[i + 1], kv1);
+      }
+      const float acc = rowgroup_sum<COLS>(acc0 + acc1);
+      if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * D + j] = acc;
+    }
+  }
+  if (on) {
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (i < nrow) Sg[(size_t)i * D] = col[i];
+  }
+}
+
+template <int R, int RGS>
+__global__ __launch_bounds__(64) void delta_scan_cols_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                             const float* __restrict__ v, int ldv,
+                                                             const float* __restrict__ decay, const float* __restrict__ beta,
+                                                             float* __restrict__ state, const int* __restrict__ cu,
+                                                             const int* __restrict__ slots, float* __restrict__ out, int H,
+                                                             int G, int DK, int DV) {
+  constexpr int COLS = 64 / RGS, NP = kTB * RGS * R / 64, LD = RGS * R + RGS;
+  extern __shared__ float lds[];
+  const int h = blockIdx.x, s = blockIdx.y, cb = blockIdx.z, lane = threadIdx.x;
+  const int jj = lane % COLS, rg = lane / COLS, j = cb * COLS + jj;
+  const bool on = j < DV;
+  const int row0 = rg * R, nrow = max(0, min(R, DK - row0));
+  const int g = h / (H / G);
+  float* qs = lds;
+  float* ks = qs + kTB * LD;
+  float* gs = ks + kTB * LD;
+  float* vs = gs + kTB * LD;     // [kTB][COLS]
+  float* bs = vs + kTB * COLS;   // [kTB]
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;
+  for (int x = lane; x < 3 * kTB * LD; x += 64) lds[x] = 0.f;
+  float* Sg = state + (((size_t)slots[s] * H + h) * DK + row0) * DV + j;
+  float col[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) col[i] = (on && i < nrow) ? Sg[(size_t)i * DV] : 0.f;
+  float pq[NP], pk[NP], pg[NP], pv[2], pb = 0.f;
+  auto fetch = [&](int tb) {
+    const int n = min(kTB, t1 - tb);
+#pragma unroll
+    for (int x = 0; x < NP; ++x) {
+      const int idx = x * 64 + lane, tt = idx / DK, i = idx - tt * DK;
+      if (tt < n) {
+        pq[x] = q[((size_t)(tb + tt) * G + g) * DK + i];
+        pk[x] = k[((size_t)(tb + tt) * G + g) * DK + i];
+        pg[x] = decay[((size_t)(tb + tt) * H + h) * DK + i];
+      }
+    }
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+      const int idx = x * 64 + lane, tt = idx / COLS, c = cb * COLS + idx % COLS;
+      pv[x] = (tt < n && c < DV) ? v[(size_t)(tb + tt) * ldv + (size_t)h * DV + c] : 0.f;
+    }
+    if (lane < n) pb = beta[(size_t)(tb + lane) * H + h];
+  };
+  fetch(t0);
+  for (int tb = t0; tb < t1; tb += kTB) {
+    const int n = min(kTB, t1 - tb);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int x = 0; x < NP; ++x) {
+      const int idx = x * 64 + lane, tt = idx / DK, i = idx - tt * DK;
+      if (tt < n) {
+        const int a = tt * LD + lds_row<R>(i);
+        qs[a] = pq[x];
+        ks[a] = pk[x];
+        gs[a] = pg[x];
+      }
+    }
+#pragma unroll
+    for (int x = 0; x < 2; ++x)
+      if (x * 64 + lane < kTB * COLS) vs[x * 64 + lane] = pv[x];
+    if (lane < kTB) bs[lane] = pb;
+    __builtin_amdgcn_wave_barrier();
+    if (tb + kTB < t1) fetch(tb + kTB);
+    for (int tt = 0; tt < n; ++tt) {
+      const float vj = vs[tt * COLS + jj], bt = bs[tt];
+      const int a = tt * LD + row0 + rg;
+      float m0 = 0.f, m1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < R; i += 2) {
+        col[i] *= gs[a + i];
+        col[i + 1] *= gs[a + i + 1];
+        m0 = fmaf(col[i], ks[a + i], m0);
+        m1 = fmaf(col[i + 1], ks[a + i + 1], m1);
+      }
+      const float uj = bt * (vj - rowgroup_sum<COLS>(m0 + m1));
+      float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < R; i += 2) {
+        col[i] = fmaf(ks[a + i], uj, col[i]);
+        col[i + 1] = fmaf(ks[a + i + 1], uj, col[i + 1]);
+        o0 = fmaf(col[i], qs[a + i], o0);
+        o1 = fmaf(col[i + 1], qs[a + i + 1], o1);
+      }
+      const float oo = rowgroup_sum<COLS>(o0 + o1);
+      if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * DV + j] = oo;
+    }
+  }
+  if (on) {
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (i < nrow) Sg[(size_t)i * DV] = col[i];
+  }
+}
+
 }  // namespace
 
 void gai_token_shift_mix(const void* h, const float* mu, int NM, const float* shift_state, const int* cu,
@@ -290,9 +492,27 @@ void gai_conv_silu(const void* x, int ldx, const float* w, const float* state, c
 }
 
 void gai_wkv_scan(const void* r, const void* k, const void* v, int ld, const float* wpre, const float* w0,
-                  const float* u, float* state, const int* cu, const int* slots, int S, float* out, int H, int D,
+                  const float* u, float* state, const int* cu, const int* slots, int S, int T, float* out, int H, int D,
                   int dt, hipStream_t st) {
   if (S == 0) return;
+  if (D > kMaxDK) gai_launch_error(__FILE__, __LINE__, "wkv_scan: head size above 256");
+  if (T > S) {  // some sequence brings more than one row: the column-sliced scan
+#define GAI_WKV(TA, R, RGS)                                                                                          \
+  do {                                                                                                               \
+    const dim3 grid(H, S, (D + 64 / RGS - 1) / (64 / RGS));                                                          \
+    const size_t lds = (size_t)(3 * kTB * (RGS * R + RGS) + kTB * (64 / RGS)) * sizeof(float);                       \
+    wkv_scan_cols_kernel<TA, R, RGS><<<grid, 64, lds, st>>>((const TA*)r, (const TA*)k, (const TA*)v, ld, wpre, w0, \
+                                                            u, state, cu, slots, out, H, D);                        \
+  } while (0)
+    if (dt) {
+      if (D <= 64) GAI_WKV(float, 16, 4); else if (D <= 128) GAI_WKV(float, 16, 8); else GAI_WKV(float, 32, 8);
+    } else {
+      if (D <= 64) GAI_WKV(bf16, 16, 4); else if (D <= 128) GAI_WKV(bf16, 16, 8); else GAI_WKV(bf16, 32, 8);
+    }
+#undef GAI_WKV
+    GAI_LAUNCH_CHECK();
+    return;
+  }
   const int RG = (D + kRows - 1) / kRows;
   if (D > kMaxDK || D * RG > 1024) gai_launch_error(__FILE__, __LINE__, "wkv_scan: head size above 256");
   const dim3 grid(H, S);
@@ -320,9 +540,24 @@ void gai_delta_prep(const float* qkv, int ld, const void* a, int lda, const void
 }
 
 void gai_delta_scan(const float* q, const float* k, const float* v, int ldv, const float* decay, const float* beta,
-                    float* state, const int* cu, const int* slots, int S, float* out, int H, int G, int DK, int DV,
-                    hipStream_t st) {
+                    float* state, const int* cu, const int* slots, int S, int T, float* out, int H, int G, int DK,
+                    int DV, hipStream_t st) {
   if (S == 0) return;
+  if (H % G) gai_launch_error(__FILE__, __LINE__, "delta_scan: heads must be a multiple of key heads");
+  if (DK > kMaxDK) gai_launch_error(__FILE__, __LINE__, "delta_scan: key head size above 256");
+  if (T > S) {  // some sequence brings more than one row: the column-sliced scan
+#define GAI_DELTA(R, RGS)                                                                                            \
+  do {                                                                                                               \
+    const dim3 grid(H, S, (DV + 64 / RGS - 1) / (64 / RGS));                                                         \
+    const size_t lds = (size_t)(3 * kTB * (RGS * R + RGS) + kTB * (64 / RGS) + kTB) * sizeof(float);                 \
+    delta_scan_cols_kernel<R, RGS><<<grid, 64, lds, st>>>(q, k, v, ldv, decay, beta, state, cu, slots, out, H, G,   \
+                                                          DK, DV);                                                   \
+  } while (0)
+    if (DK <= 64) GAI_DELTA(16, 4); else if (DK <= 128) GAI_DELTA(16, 8); else GAI_DELTA(32, 8);
+#undef GAI_DELTA
+    GAI_LAUNCH_CHECK();
+    return;
+  }
   const int RG = (DK + kRows - 1) / kRows;
   if (DK > kMaxDK || DV * RG > 1024) gai_launch_error(__FILE__, __LINE__, "delta_scan: head sizes above 256");
   if (H % G) gai_launch_error(__FILE__, __LINE__, "delta_scan: heads must be a multiple of key heads");

@@ -39,6 +39,7 @@ import torch
 import torch.nn.functional as F
 
 from .. import ops
+from ..engine.state_pool import StatePool
 from ..parallel.dist import DistContext, get_context
 from .common import ForwardBatch, randn_like_
 
@@ -182,6 +183,8 @@ def _l2n(x, eps=1e-6):
 class Qwen3NextModel:
     """Weights (plain tensors) + forward for the serving engine (same hooks as LlamaModel / Mllama)."""
 
+    has_recurrent_state = True  # no prefix-cache reuse: cached prefix pages carry no linear-attention state
+
     def __init__(self, cfg: Qwen3NextConfig, device=None, dtype=torch.bfloat16, dist_ctx: DistContext | None = None,
                  state_slots: Optional[int] = None):
         self.cfg = cfg
@@ -208,10 +211,9 @@ class Qwen3NextModel:
         self._alloc()
         # linear-attention state pool (allocated on first use): slot -> conv window + recurrent state
         self.n_slots = state_slots or int(os.environ.get("GAI_LINEAR_STATE_SLOTS", "64"))
+        self.pool = StatePool(self.n_slots, self.device)  # slot accounting shared with the other state-slot models
         self.conv_state: Optional[torch.Tensor] = None  # [Ll, slots + 1, K - 1, conv_dim] fp32
         self.ssm_state: Optional[torch.Tensor] = None   # [Ll, slots + 1, Hv, dk, dv] fp32 (last slot = pad)
-        self.slot_of: Dict[int, int] = {}
-        self.free_slots: List[int] = []
 
     # ------------------------------------------------------------------ rope (partial, permuted)
     @staticmethod
@@ -371,33 +373,24 @@ class Qwen3NextModel:
     def _ensure_pool(self):
         if self.ssm_state is not None:
             return
-        c, Ll, n = self.cfg, len(self.lin_layers), self.n_slots + 1
-        self.conv_state = torch.zeros(Ll, n, c.linear_conv_kernel_dim - 1, self.conv_dim, device=self.device)
-        self.ssm_state = torch.zeros(Ll, n, c.linear_num_value_heads, c.linear_key_head_dim,
-                                     c.linear_value_head_dim, device=self.device)
-        self.free_slots = list(range(self.n_slots))[::-1]
+        c, Ll = self.cfg, len(self.lin_layers)
+        self.conv_state = self.pool.add("conv", (Ll, c.linear_conv_kernel_dim - 1, self.conv_dim), slot_dim=1)
+        self.ssm_state = self.pool.add("ssm", (Ll, c.linear_num_value_heads, c.linear_key_head_dim,
+                                               c.linear_value_head_dim), slot_dim=1)
 
     @property
     def pad_slot(self) -> int:
         return self.n_slots
 
     def _slot(self, sid: int, fresh: bool) -> int:
-        s = self.slot_of.get(sid)
-        if s is None:
-            if not self.free_slots:
-                raise RuntimeError("Qwen3-Next state pool exhausted: raise GAI_LINEAR_STATE_SLOTS or lower "
-                                   "max_num_seqs")
-            s = self.slot_of[sid] = self.free_slots.pop()
-            fresh = True
-        if fresh:
-            self.conv_state[:, s].zero_()
-            self.ssm_state[:, s].zero_()
-        return s
+        return self.pool.slot(sid, fresh)
+
+    @property
+    def slot_of(self) -> Dict[int, int]:
+        return self.pool.slot_of
 
     def release_request(self, sid: int):
-        s = self.slot_of.pop(sid, None)
-        if s is not None:
-            self.free_slots.append(s)
+        self.pool.release(sid)
 
     def prepare_batch(self, fb: ForwardBatch):
         """Engine hook: map the step's sequences to state slots (fresh prompts start from zero state)."""
