@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
     const TA* __restrict__ q, const TA* __restrict__ k_cache, const TA* __restrict__ v_cache,
     const int* __restrict__ block_tables, int maxb, const int* __restrict__ cu_q, const int* __restrict__ ctx, int S,
     TA* __restrict__ out, int TH, int H, int G, int DK, int DV, float scale, float softcap, int window,
-    const float* __restrict__ r1, const float* __restrict__ r2, const TA* __restrict__ gate, int ldg) {
+    const float* __restrict__ r1, const float* __restrict__ r2, const TA* __restrict__ gate, int ldg, int skip_len) {
   extern __shared__ float lds[];
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int th = blockIdx.x * 4 + wid;
@@ -139,6 +139,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
     if (cu_q[mid] <= t) lo = mid; else hi = mid;
   }
   const int s = lo, c0 = cu_q[s];
+  if (cu_q[s + 1] - c0 >= skip_len) return;  // long portions run on the matrix-core kernel
   const int pos = ctx[s] - (cu_q[s + 1] - c0) + (t - c0);
   const int first = window > 0 ? max(0, pos - window + 1) : 0;
   const TA* qr = q + (size_t)th * DK;
@@ -195,6 +196,162 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
   }
 }
 
+// ---- prompt portions in bf16: query tiles on the matrix cores ------------------------------------------------------
+// One wave64 per (32 consecutive queries of a sequence, head); the 4 waves of a workgroup take 4 neighbouring heads of
+// the same tile, so with GQA their K / V reads meet in L1. S^T = K.Q^T on v_mfma_f32_32x32x16_bf16 leaves one query per
+// lane (both lane halves hold 16 of the block's 32 keys), so cap, distance penalty and the online softmax are
+// in-register fp32. P.V runs on the same MFMA with the fp32 weights split into two bf16 terms (p = hi + lo, relative
+// error 2^-17: below one rounding of the bf16 values they multiply), accumulated in fp32. K rows and V^T page rows are
+// read straight from the paged cache into MFMA fragments (16-byte / 8-byte loads; the key order inside a 16-key step is
+// the accumulator's row order, so no shuffle is needed between the two products).
+typedef __bf16 bf16x4v __attribute__((ext_vector_type(4)));
+constexpr int kTileQ = 32;
+constexpr int kMfmaMinLen = 8;   // shorter portions (and decoded tokens) stay on the one-wave-per-row kernel
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kMasked = -1e30f;
+
+__device__ __forceinline__ float max_halves(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_halves(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// tanh through one v_exp_f32 and one reciprocal; a short odd polynomial where the quotient form would cancel
+__device__ __forceinline__ float tanh_fast(float y) {
+  const float e = __builtin_amdgcn_exp2f(2.0f * kLog2e * y);
+  const float big = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);
+  const float y2 = y * y;
+  const float small = y * (1.0f + y2 * (-0.33333334f + y2 * (0.13333334f - 0.053968254f * y2)));
+  return fabsf(y) < 0.25f ? small : big;
+}
+
+template <int DK, int DV>
+__global__ __launch_bounds__(256) void window_attention_mfma_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+    const int* __restrict__ block_tables, int maxb, const int* __restrict__ cu_q, const int* __restrict__ ctx, int S,
+    bf16* __restrict__ out, int H, int G, float scale, float softcap, int window, const float* __restrict__ r1,
+    const float* __restrict__ r2, const bf16* __restrict__ gate, int ldg) {
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int h = blockIdx.y * 4 + wid;
+  if (h >= H) return;
+  // tile -> (sequence, first row): sequences of at least kMfmaMinLen rows own ceil(len / 32) tiles each
+  int s = 0, seen = 0, len = 0;
+  for (; s < S; ++s) {
+    len = cu_q[s + 1] - cu_q[s];
+    const int nt = len >= kMfmaMinLen ? (len + kTileQ - 1) / kTileQ : 0;
+    if ((int)blockIdx.x < seen + nt) break;
+    seen += nt;
+  }
+  if (s == S) return;
+  const int row0 = ((int)blockIdx.x - seen) * kTileQ, nrows = min(kTileQ, len - row0);
+  const int qi = lane & 31, hb = lane >> 5, g = h / (H / G);
+  const bool valid = qi < nrows;
+  const int t = cu_q[s] + row0 + min(qi, nrows - 1);
+  const int pos0 = ctx[s] - len + row0;             // position of the tile's first query
+  const int pos = pos0 + min(qi, nrows - 1), last = pos0 + nrows - 1;
+  const int first = window > 0 ? max(0, pos0 - window + 1) : 0;
+  const int* bt = block_tables + (size_t)s * maxb;
+  bf16x8 qf[DK / 16];
+  const bf16* qr = q + ((size_t)t * H + h) * DK + 8 * hb;
+#pragma unroll
+  for (int i = 0; i < DK / 16; ++i) qf[i] = load8(qr + 16 * i);
+  f32x16 acc_o[DV / 32];
+#pragma unroll
+  for (int i = 0; i < DV / 32; ++i) acc_o[i] = f32x16{};
+  float m_run = kMasked, l_run = 0.f;
+  const float b1 = r1 ? r1[h] : 0.f, b2 = r1 ? r2[h] : 0.f;
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+  for (int kb = first & ~31; kb <= last; kb += 32) {
+    // ---- S^T block: rows = keys kb .. kb + 31, columns = the tile's queries
+    const int kn = min(kb + qi, last);  // keys past the tile's last position: any valid row (masked below)
+    const bf16* kr = k_cache + (((size_t)bt[kn >> 4] * G + g) * 16 + (kn & 15)) * DK + 8 * hb;
+    f32x16 sc = f32x16{};
+#pragma unroll
+    for (int i = 0; i < DK / 16; ++i) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load8(kr + 16 * i), qf[i], sc, 0, 0, 0);
+    float mt = kMasked;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int dist = pos - (kb + (r & 3) + 8 * (r >> 2) + 4 * hb);
+      float x = sc[r] * scale;
+      if (softcap > 0.f) x = softcap * tanh_fast(x * inv_cap);
+      if (r1) x -= b1 * (0.6931471805599453f * __builtin_amdgcn_logf(fmaf(b2, (float)max(dist, 0), 1.0f)));
+      const bool ok = valid && dist >= 0 && (window <= 0 || dist < window);
+      x = ok ? x : kMasked;
+      sc[r] = x;
+      mt = fmaxf(mt, x);
+    }
+    mt = max_halves(mt);
+    const float m_new = fmaxf(m_run, mt);
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * kLog2e);
+    m_run = m_new;
+    float rs = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float p = sc[r] > 0.5f * kMasked ? __builtin_amdgcn_exp2f((sc[r] - m_new) * kLog2e) : 0.f;
+      sc[r] = p;
+      rs += p;
+    }
+    l_run = l_run * alpha + rs;
+#pragma unroll
+    for (int i = 0; i < DV / 32; ++i) acc_o[i] *= alpha;
+    // ---- O^T += V^T . P^T, one 16-key page per step
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int kp = kb + 16 * ks;
+      if (kp > last) break;
+      bf16x8 ph, pl;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float p = sc[8 * ks + e];
+        ph[e] = (bf16)p;
+        pl[e] = (bf16)(p - (float)ph[e]);
+      }
+      const bf16* vr = v_cache + (((size_t)bt[kp >> 4] * G + g) * DV + qi) * 16 + 4 * hb;
+#pragma unroll
+      for (int i = 0; i < DV / 32; ++i) {
+        const bf16x4v a = *reinterpret_cast<const bf16x4v*>(vr + (size_t)32 * i * 16);
+        const bf16x4v b = *reinterpret_cast<const bf16x4v*>(vr + (size_t)32 * i * 16 + 8);
+        const bf16x8 vf = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+        acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, ph, acc_o[i], 0, 0, 0);
+        acc_o[i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pl, acc_o[i], 0, 0, 0);
+      }
+    }
+  }
+  const float l = sum_halves(l_run);
+  if (!valid) return;
+  const float inv_l = 1.0f / l;
+  bf16* o = out + ((size_t)t * H + h) * DV;
+  const bf16* gr = gate ? gate + (size_t)t * ldg + (size_t)h * DV : nullptr;
+#pragma unroll
+  for (int i = 0; i < DV / 32; ++i) {
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      const int c = 32 * i + 8 * r4 + 4 * hb;
+      bf16x4v y;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float v = acc_o[i][4 * r4 + e] * inv_l;
+        if (gr) v *= 1.0f / (1.0f + __expf(-(float)gr[c + e]));
+        y[e] = (bf16)v;
+      }
+      *reinterpret_cast<bf16x4v*>(o + c) = y;
+    }
+  }
+}
+
+template <int DK, int DV>
+void launch_window_mfma(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int maxb,
+                        const int* cu_q, const int* ctx, int S, void* out, int T, int H, int G, float scale,
+                        float softcap, int window, const float* r1, const float* r2, const void* gate, int ldg,
+                        hipStream_t st) {
+  const dim3 grid((T + kTileQ - 1) / kTileQ + S, (H + 3) / 4);
+  window_attention_mfma_kernel<DK, DV><<<grid, 256, 0, st>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache,
+                                                             block_tables, maxb, cu_q, ctx, S, (bf16*)out, H, G, scale,
+                                                             softcap, window, r1, r2, (const bf16*)gate, ldg);
+}
+
 }  // namespace
 
 void gai_qknorm_kv_write(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* wq,
@@ -221,14 +378,29 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
   if (H % G) gai_launch_error(__FILE__, __LINE__, "window_attention: heads must be a multiple of kv heads");
   const int TH = T * H, grid = (TH + 3) / 4;
   const size_t lds = 4 * (size_t)(DK + 64) * sizeof(float);
+  // bf16 steps with prompt portions (more rows than sequences): portions of >= kMfmaMinLen rows go to the query-tiled
+  // matrix-core kernel for the head sizes it is instantiated for; the rest runs below
+  int skip_len = 0x7fffffff;
+  if (!dt && T > S && (!gate || ldg % 4 == 0)) {
+#define GAI_WIN(K_, V_)                                                                                              \
+  if (DK == K_ && DV == V_) {                                                                                        \
+    launch_window_mfma<K_, V_>(q, k_cache, v_cache, block_tables, maxb, cu_q, ctx, S, out, T, H, G, scale, softcap,   \
+                               window, r1, r2, gate, ldg, st);                                                        \
+    skip_len = kMfmaMinLen;                                                                                          \
+  }
+    GAI_WIN(64, 64) GAI_WIN(64, 128) GAI_WIN(128, 64) GAI_WIN(128, 128) GAI_WIN(256, 256)
+#undef GAI_WIN
+    GAI_LAUNCH_CHECK();
+  }
   if (dt)
     window_attention_kernel<float><<<grid, 256, lds, st>>>((const float*)q, (const float*)k_cache,
                                                            (const float*)v_cache, block_tables, maxb, cu_q, ctx, S,
                                                            (float*)out, TH, H, G, DK, DV, scale, softcap, window, r1, r2,
-                                                           (const float*)gate, ldg);
+                                                           (const float*)gate, ldg, skip_len);
   else
     window_attention_kernel<bf16><<<grid, 256, lds, st>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache,
                                                           block_tables, maxb, cu_q, ctx, S, (bf16*)out, TH, H, G, DK,
-                                                          DV, scale, softcap, window, r1, r2, (const bf16*)gate, ldg);
+                                                          DV, scale, softcap, window, r1, r2, (const bf16*)gate, ldg,
+                                                          skip_len);
   GAI_LAUNCH_CHECK();
 }

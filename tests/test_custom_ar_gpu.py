@@ -15,7 +15,10 @@ pytestmark = [pytest.mark.gpu, pytest.mark.multirank]
 
 @pytest.mark.parametrize("world", [2, 4, 8])
 def test_custom_allreduce_matches_sum(tmp_path, world, gpu_box):
-    run = M.run_ranks(W.custom_ar_worker, world, (M.free_port(), str(tmp_path)), 100)
+    # 8 ranks share one GPU's hardware queues: every step waits for all eight kernels to be resident together, so the
+    # wall time grows much faster than the rank count (the 2- and 4-rank runs take 10 - 20 s)
+    run = M.run_ranks(W.custom_ar_worker, world, (M.free_port(), str(tmp_path)), 100 if world < 8 else 240)
+    print(f"world {world}: ranks joined after {run.elapsed:.0f} s")
     pr = M.assert_coresident(tmp_path, "car", world, run)
     assert not any(run.late), f"ranks still running at the deadline: {run.late}; census {run.peak}"
     assert all(c == 0 for c in run.exitcodes), run.exitcodes

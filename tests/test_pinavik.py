@@ -205,11 +205,11 @@ def test_far_token_through_state(device, dtype):
     assert rel_err(got["a"][-1:], wa) < tol(dtype) and rel_err(got["b"][-1:], wb) < tol(dtype)
 
 
-def _attention_probe(device, dtype, window, n_ctx, hot, portion):
+def _attention_probe(device, dtype, window, n_ctx, hot, portion, dk=8, dv=16):
     """ops-level: one head, keys of n_ctx positions through the paged cache (pages deliberately scattered); the key at
     position `hot` is aligned with the last query and scaled up so that its score stands out; returns the last query's
     output. Values are one-hot in the position (mod 16), so the output tells which keys were seen."""
-    dk, dv, B = 8, 16, ops.BLOCK
+    B = ops.BLOCK
     dev = torch.device(device)
     nb = (n_ctx + B - 1) // B
     pages = list(range(nb + 3))[::-1][:nb]  # not the identity
@@ -222,7 +222,7 @@ def _attention_probe(device, dtype, window, n_ctx, hot, portion):
     k = k - torch.outer(k @ qh, qh)  # every other key is orthogonal to the last query: score 0
     k[hot] = q_last * 3.0
     v = torch.zeros(n_ctx, dv)
-    v[torch.arange(n_ctx), torch.arange(n_ctx) % dv] = 1.0
+    v[torch.arange(n_ctx), torch.arange(n_ctx) % 16] = 1.0
     v[hot] = 0.0
     v[hot, 5] = -7.0
     q = torch.randn(n_ctx, dk, generator=g)
@@ -256,6 +256,39 @@ def test_window_edges_and_page_borders(device, dtype, portion):
         assert outside[5] > -1e-6 and abs(outside.sum().item() - 1.0) < 1e-4, (window, outside)
     for hot in (15, 16, 31, 32, 0):
         assert _attention_probe(device, dtype, 400, 330, hot, portion if portion != [1] else [300, 1])[5] < -3.0, hot
+
+
+@_GPU
+@pytest.mark.parametrize("dk,dv", [(64, 64), (128, 64), (64, 128), (128, 128), (256, 256)])
+def test_window_edges_matrix_core_kernel(dk, dv):
+    """The same stand-out key probes on the bf16 query-tiled matrix-core kernel (head sizes it is built for, portions of
+    8 rows and more), beside shorter portions that stay on the one-wave-per-row kernel."""
+    n, dt = 150, torch.bfloat16
+    for portion in ([1000], [70, 40, 9, 31], [120, 3, 27]):
+        for window in (5, 32, 33, 64, 100):
+            inside = _attention_probe("cuda", dt, window, n, n - window, portion, dk, dv)
+            outside = _attention_probe("cuda", dt, window, n, n - window - 1, portion, dk, dv)
+            assert inside[5] < -3.0, (portion, window, inside)
+            assert outside[5] > -1e-6 and abs(outside.sum().item() - 1.0) < 2e-2, (portion, window, outside)
+        for hot in (15, 16, 31, 32, 63, 64, 0):
+            assert _attention_probe("cuda", dt, 400, 330, hot, [200, 130], dk, dv)[5] < -3.0, hot
+
+
+@_GPU
+def test_matrix_core_attention_in_model():
+    """bf16 model with 64- and 128-wide heads: portions of 8+ rows take the matrix-core attention kernel, shorter ones
+    and decoded tokens the row kernel; both against the oracle, alone and in a mixed batch."""
+    layers = [O.with_mlp(O.att(dim=64, vdim=64, heads=4, kv_heads=2, window=40)), O.with_mlp(O.wkv(dim=16, heads=4)),
+              O.with_mlp(O.att(dim=128, vdim=64, heads=2, kv_heads=1, window=70, softcap=8.0))]
+    cfg = O.make_config(layers, width=128, vocab=128, loop=(0, 2, 2))
+    sd = O.random_checkpoint(cfg, 61)
+    prompts = {"a": tokens(150, 128, 62), "b": tokens(90, 128, 63)}
+    want = {n: O.forward(cfg, sd, t) for n, t in prompts.items()}
+    eng = make_engine(cfg, sd, "cuda", torch.bfloat16)
+    sched = [[("a", 70)], [("a", 33), ("b", 50)], [("a", 9), ("b", 1)], [("a", 1), ("b", 39)], [("a", 37)]]
+    got = run_schedule(eng, prompts, sched)
+    for n in prompts:
+        assert close(got[n], want[n], torch.bfloat16), n
 
 
 # ------------------------------------------------------------------------------------------- shapes of other models
