@@ -172,7 +172,7 @@ void conv_silu(const Tensor& x, const Tensor& w, const Tensor& state, const Tens
 }
 
 void wkv_scan(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& wpre, const Tensor& w0, const Tensor& u,
-              Tensor& state, const Tensor& cu, const Tensor& slots, Tensor& out) {
+              Tensor& state, const Tensor& cu, const Tensor& slots, Tensor& out, const optional<Tensor>& ws) {
   const int dt = act_dt(r, "r");
   same_dt(k, dt, "k");
   same_dt(v, dt, "v");
@@ -185,8 +185,14 @@ void wkv_scan(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& w
   TORCH_CHECK(k.size(0) == T && v.size(0) == T && wpre.numel() == (int64_t)T * H * D && w0.numel() == H * D &&
                   u.numel() == H * D && cu.numel() == S + 1 && out.numel() == (int64_t)T * H * D,
               "wkv_scan: decay / bonus / cu / out shapes");
+  float* wsp = nullptr;  // scratch for the decays of a step with prompt portions (absent: the per-sequence kernel runs)
+  if (ws) {
+    TORCH_CHECK(ws->is_cuda() && ws->scalar_type() == at::kFloat && ws->is_contiguous() && ws->numel() >= wpre.numel(),
+                "wkv_scan: workspace must be fp32 [T, H * D]");
+    wsp = ws->data_ptr<float>();
+  }
   gai_wkv_scan(r.data_ptr(), k.data_ptr(), v.data_ptr(), ld, f32(wpre, "wpre"), f32(w0, "w0"), f32(u, "u"),
-               f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, T, f32w(out, "out"), H, D, dt, cur_stream());
+               f32w(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S, T, f32w(out, "out"), H, D, dt, wsp, cur_stream());
 }
 
 void delta_prep(const Tensor& qkv, const Tensor& a, const Tensor& b, const Tensor& A_log, const Tensor& dt_bias,

@@ -225,7 +225,7 @@ void gai_conv_silu(const void* x, int ldx, const float* w, const float* state, c
                    float* y, int T, int C, int K, int dt, hipStream_t st);
 void gai_wkv_scan(const void* r, const void* k, const void* v, int ld, const float* wpre, const float* w0,
                   const float* u, float* state, const int* cu, const int* slots, int S, int T, float* out, int H, int D,
-                  int dt, hipStream_t st);
+                  int dt, float* ws, hipStream_t st);
 void gai_delta_prep(const float* qkv, int ld, const void* a, int lda, const void* b, int ldb, const float* A_log,
                     const float* dt_bias, float* qn, float* kn, float* decay, float* beta, int T, int H, int G, int DK,
                     int dt, hipStream_t st);

@@ -257,33 +257,51 @@ __global__ __launch_bounds__(1024) void delta_scan_kernel(const float* __restric
 
 // ---- prompt portions: one wave64 per (head, sequence, block of state columns) -------------------------------------
 // The columns of S evolve independently of each other, so a long portion is spread over many waves per head instead
-// of one workgroup: lane (rg, jj) owns rows [rg R, rg R + R) of column jj (RGS row groups x 64 / RGS columns), the token
-// inputs of 8 tokens at a time are staged in LDS by the wave itself (coalesced loads, prefetched into registers one
-// round ahead), and the row-group reductions are lane shuffles: no workgroup barrier anywhere in the token loop. LDS
+// of one workgroup: lane (jj, rg) owns rows [rg R, rg R + R) of column jj (64 / RGS columns x RGS row groups), the token
+// inputs of 8 tokens at a time are staged in LDS by the wave itself (prefetched into registers one round ahead), and
+// the row-group reductions are DPP adds: no workgroup barrier and no LDS shuffle anywhere in the token loop. LDS
 // rows past DK stay zero, so the token loop has no row guard (branch-free: its LDS reads are issued in batches).
 constexpr int kTB = 8;
 
 template <int R>
 __device__ __forceinline__ int lds_row(int row) { return row + row / R; }  // row groups land in different banks
 
-template <int COLS>
+// Sum over the RGS row groups of a column, in every lane of the group. The row groups of one column sit in RGS
+// neighbouring lanes (RGS <= 16: inside one DPP row), so the butterfly is 2 - 4 v_add_f32 with DPP operands (quad
+// permutes, then half-row and row mirrors - the mirrored partner holds its group's total in every lane) and never
+// goes through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int RGS>
 __device__ __forceinline__ float rowgroup_sum(float v) {
-#pragma unroll
-  for (int o = COLS; o < 64; o <<= 1) v += __shfl_xor(v, o, 64);
+  static_assert(RGS == 4 || RGS == 8 || RGS == 16, "row groups of one column share a DPP row");
+  v += dpp_f<0xB1>(v);                       // quad_perm [1, 0, 3, 2]
+  v += dpp_f<0x4E>(v);                       // quad_perm [2, 3, 0, 1]
+  if (RGS >= 8) v += dpp_f<0x141>(v);        // row_half_mirror
+  if (RGS >= 16) v += dpp_f<0x140>(v);       // row_mirror
   return v;
+}
+
+// decay of every (token, head, channel) ahead of the serial scan: exp(-exp(wpre + w0)), token-parallel
+__global__ __launch_bounds__(256) void wkv_decay_kernel(const float* __restrict__ wpre, const float* __restrict__ w0,
+                                                        float* __restrict__ wdecay, size_t n, int HD) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n) wdecay[i] = expf(-expf(wpre[i] + w0[i % HD]));
 }
 
 template <typename TA, int R, int RGS>
 __global__ __launch_bounds__(64) void wkv_scan_cols_kernel(const TA* __restrict__ r, const TA* __restrict__ k,
-                                                           const TA* __restrict__ v, int ld, const float* __restrict__ wpre,
-                                                           const float* __restrict__ w0, const float* __restrict__ u,
+                                                           const TA* __restrict__ v, int ld,
+                                                           const float* __restrict__ wdecay, const float* __restrict__ u,
                                                            float* __restrict__ state, const int* __restrict__ cu,
                                                            const int* __restrict__ slots, float* __restrict__ out, int H,
                                                            int D) {
   constexpr int COLS = 64 / RGS, NP = kTB * RGS * R / 64, LD = RGS * R + RGS;
   extern __shared__ float lds[];
   const int h = blockIdx.x, s = blockIdx.y, cb = blockIdx.z, lane = threadIdx.x;
-  const int jj = lane % COLS, rg = lane / COLS, j = cb * COLS + jj;
+  const int jj = lane / RGS, rg = lane % RGS, j = cb * COLS + jj;
   const bool on = j < D;
   const int row0 = rg * R, nrow = max(0, min(R, D - row0));
   float* rs = lds;
@@ -300,17 +318,21 @@ __global__ __launch_bounds__(64) void wkv_scan_cols_kernel(const TA* __restrict_
     col[i] = (on && i < nrow) ? Sg[(size_t)i * D] : 0.f;
     ur[i] = i < nrow ? u[(size_t)h * D + row0 + i] : 0.f;
   }
+  // staging map without divisions: lane = (token of the round, 1 of 8 parts); a part walks its token's row with stride 8
+  constexpr int NPART = 64 / kTB;
+  static_assert(NP * NPART >= RGS * R, "staging covers a full row");
+  const int stt = lane / NPART, spart = lane % NPART;
   float pr[NP], pk[NP], pw[NP], pv[2];
   auto fetch = [&](int tb) {
     const int n = min(kTB, t1 - tb);
 #pragma unroll
     for (int x = 0; x < NP; ++x) {
-      const int idx = x * 64 + lane, tt = idx / D, i = idx - tt * D;
-      if (tt < n) {
-        const size_t o = (size_t)(tb + tt) * ld + (size_t)h * D + i;
+      const int i = spart + NPART * x;
+      if (stt < n && i < D) {
+        const size_t o = (size_t)(tb + stt) * ld + (size_t)h * D + i;
         pr[x] = (float)r[o];
         pk[x] = (float)k[o];
-        pw[x] = wpre[((size_t)(tb + tt) * H + h) * D + i] + w0[(size_t)h * D + i];
+        pw[x] = wdecay[((size_t)(tb + stt) * H + h) * D + i];
       }
     }
 #pragma unroll
@@ -325,12 +347,12 @@ __global__ __launch_bounds__(64) void wkv_scan_cols_kernel(const TA* __restrict_
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int x = 0; x < NP; ++x) {
-      const int idx = x * 64 + lane, tt = idx / D, i = idx - tt * D;
-      if (tt < n) {
-        const int a = tt * LD + lds_row<R>(i);
+      const int i = spart + NPART * x;
+      if (stt < n && i < D) {
+        const int a = stt * LD + lds_row<R>(i);
         rs[a] = pr[x];
         ks[a] = pk[x];
-        ws[a] = expf(-expf(pw[x]));
+        ws[a] = pw[x];
       }
     }
 #pragma unroll
@@ -350,7 +372,7 @@ __global__ __launch_bounds__(64) void wkv_scan_cols_kernel(const TA* __restrict_
         col[i] = fmaf(ws[a + i], col[i], kv0);
         col[i + 1] = fmaf(ws[a + i + 1], col[i + 1], kv1);
       }
-      const float acc = rowgroup_sum<COLS>(acc0 + acc1);
+      const float acc = rowgroup_sum<RGS>(acc0 + acc1);
       if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * D + j] = acc;
     }
   }
@@ -371,7 +393,7 @@ __global__ __launch_bounds__(64) void delta_scan_cols_kernel(const float* __rest
   constexpr int COLS = 64 / RGS, NP = kTB * RGS * R / 64, LD = RGS * R + RGS;
   extern __shared__ float lds[];
   const int h = blockIdx.x, s = blockIdx.y, cb = blockIdx.z, lane = threadIdx.x;
-  const int jj = lane % COLS, rg = lane / COLS, j = cb * COLS + jj;
+  const int jj = lane / RGS, rg = lane % RGS, j = cb * COLS + jj;
   const bool on = j < DV;
   const int row0 = rg * R, nrow = max(0, min(R, DK - row0));
   const int g = h / (H / G);
@@ -387,16 +409,19 @@ __global__ __launch_bounds__(64) void delta_scan_cols_kernel(const float* __rest
   float col[R];
 #pragma unroll
   for (int i = 0; i < R; ++i) col[i] = (on && i < nrow) ? Sg[(size_t)i * DV] : 0.f;
+  constexpr int NPART = 64 / kTB;
+  static_assert(NP * NPART >= RGS * R, "staging covers a full row");
+  const int stt = lane / NPART, spart = lane % NPART;
   float pq[NP], pk[NP], pg[NP], pv[2], pb = 0.f;
   auto fetch = [&](int tb) {
     const int n = min(kTB, t1 - tb);
 #pragma unroll
     for (int x = 0; x < NP; ++x) {
-      const int idx = x * 64 + lane, tt = idx / DK, i = idx - tt * DK;
-      if (tt < n) {
-        pq[x] = q[((size_t)(tb + tt) * G + g) * DK + i];
-        pk[x] = k[((size_t)(tb + tt) * G + g) * DK + i];
-        pg[x] = decay[((size_t)(tb + tt) * H + h) * DK + i];
+      const int i = spart + NPART * x;
+      if (stt < n && i < DK) {
+        pq[x] = q[((size_t)(tb + stt) * G + g) * DK + i];
+        pk[x] = k[((size_t)(tb + stt) * G + g) * DK + i];
+        pg[x] = decay[((size_t)(tb + stt) * H + h) * DK + i];
       }
     }
 #pragma unroll
@@ -412,9 +437,9 @@ __global__ __launch_bounds__(64) void delta_scan_cols_kernel(const float* __rest
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int x = 0; x < NP; ++x) {
-      const int idx = x * 64 + lane, tt = idx / DK, i = idx - tt * DK;
-      if (tt < n) {
-        const int a = tt * LD + lds_row<R>(i);
+      const int i = spart + NPART * x;
+      if (stt < n && i < DK) {
+        const int a = stt * LD + lds_row<R>(i);
         qs[a] = pq[x];
         ks[a] = pk[x];
         gs[a] = pg[x];
@@ -437,7 +462,7 @@ __global__ __launch_bounds__(64) void delta_scan_cols_kernel(const float* __rest
         m0 = fmaf(col[i], ks[a + i], m0);
         m1 = fmaf(col[i + 1], ks[a + i + 1], m1);
       }
-      const float uj = bt * (vj - rowgroup_sum<COLS>(m0 + m1));
+      const float uj = bt * (vj - rowgroup_sum<RGS>(m0 + m1));
       float o0 = 0.f, o1 = 0.f;
 #pragma unroll
       for (int i = 0; i < R; i += 2) {
@@ -446,7 +471,7 @@ __global__ __launch_bounds__(64) void delta_scan_cols_kernel(const float* __rest
         o0 = fmaf(col[i], qs[a + i], o0);
         o1 = fmaf(col[i + 1], qs[a + i + 1], o1);
       }
-      const float oo = rowgroup_sum<COLS>(o0 + o1);
+      const float oo = rowgroup_sum<RGS>(o0 + o1);
       if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * DV + j] = oo;
     }
   }
@@ -493,21 +518,23 @@ void gai_conv_silu(const void* x, int ldx, const float* w, const float* state, c
 
 void gai_wkv_scan(const void* r, const void* k, const void* v, int ld, const float* wpre, const float* w0,
                   const float* u, float* state, const int* cu, const int* slots, int S, int T, float* out, int H, int D,
-                  int dt, hipStream_t st) {
+                  int dt, float* ws, hipStream_t st) {
   if (S == 0) return;
   if (D > kMaxDK) gai_launch_error(__FILE__, __LINE__, "wkv_scan: head size above 256");
-  if (T > S) {  // some sequence brings more than one row: the column-sliced scan
+  if (T > S && ws) {  // some sequence brings more than one row: the column-sliced scan (ws: [T, H * D] decays)
+    const size_t nw = (size_t)T * H * D;
+    wkv_decay_kernel<<<(unsigned)((nw + 255) / 256), 256, 0, st>>>(wpre, w0, ws, nw, H * D);
 #define GAI_WKV(TA, R, RGS)                                                                                          \
   do {                                                                                                               \
     const dim3 grid(H, S, (D + 64 / RGS - 1) / (64 / RGS));                                                          \
     const size_t lds = (size_t)(3 * kTB * (RGS * R + RGS) + kTB * (64 / RGS)) * sizeof(float);                       \
-    wkv_scan_cols_kernel<TA, R, RGS><<<grid, 64, lds, st>>>((const TA*)r, (const TA*)k, (const TA*)v, ld, wpre, w0, \
-                                                            u, state, cu, slots, out, H, D);                        \
+    wkv_scan_cols_kernel<TA, R, RGS><<<grid, 64, lds, st>>>((const TA*)r, (const TA*)k, (const TA*)v, ld, ws, u,    \
+                                                            state, cu, slots, out, H, D);                           \
   } while (0)
     if (dt) {
-      if (D <= 64) GAI_WKV(float, 16, 4); else if (D <= 128) GAI_WKV(float, 16, 8); else GAI_WKV(float, 32, 8);
+      if (D <= 64) GAI_WKV(float, 8, 8); else if (D <= 128) GAI_WKV(float, 8, 16); else GAI_WKV(float, 16, 16);
     } else {
-      if (D <= 64) GAI_WKV(bf16, 16, 4); else if (D <= 128) GAI_WKV(bf16, 16, 8); else GAI_WKV(bf16, 32, 8);
+      if (D <= 64) GAI_WKV(bf16, 8, 8); else if (D <= 128) GAI_WKV(bf16, 8, 16); else GAI_WKV(bf16, 16, 16);
     }
 #undef GAI_WKV
     GAI_LAUNCH_CHECK();
@@ -553,7 +580,7 @@ void gai_delta_scan(const float* q, const float* k, const float* v, int ldv, con
     delta_scan_cols_kernel<R, RGS><<<grid, 64, lds, st>>>(q, k, v, ldv, decay, beta, state, cu, slots, out, H, G,   \
                                                           DK, DV);                                                   \
   } while (0)
-    if (DK <= 64) GAI_DELTA(16, 4); else if (DK <= 128) GAI_DELTA(16, 8); else GAI_DELTA(32, 8);
+    if (DK <= 64) GAI_DELTA(8, 8); else if (DK <= 128) GAI_DELTA(8, 16); else GAI_DELTA(16, 16);
 #undef GAI_DELTA
     GAI_LAUNCH_CHECK();
     return;

@@ -254,7 +254,8 @@ class PinavikModel:
                 w[x + "mu"] = torch.stack([f32(sd[x + "mu." + s]) for s in "rkvgw"])
                 for k in "rkvg":
                     w[x + k] = mat(sd[x + k])
-                w[x + "w1"], w[x + "w2"] = mat(sd[x + "w1"]), mat(sd[x + "w2"])
+                # w2 multiplies the fp32 tanh output: kept fp32 so that the fp32 product converts nothing per step
+                w[x + "w1"], w[x + "w2"] = mat(sd[x + "w1"]), f32(sd[x + "w2"])
                 for k in ("w0", "u", "norm"):
                     w[x + k] = f32(sd[x + k]).reshape(-1)
             else:

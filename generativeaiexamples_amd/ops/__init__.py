@@ -1134,7 +1134,9 @@ def wkv_scan(r, k, v, wpre, w0, u, state, cu, slots):
         return ref.wkv_scan(r, k, v, wpre, w0, u, state, cu, slots)
     H, D = state.shape[1], state.shape[2]
     out = torch.empty(r.shape[0], H, D, dtype=torch.float32, device=r.device)
-    native().wkv_scan(r, k, v, wpre, w0, u, state, cu, slots, out)
+    # a step with prompt portions (more rows than sequences) precomputes the decays token-parallel into a scratch
+    ws = torch.empty_like(wpre) if r.shape[0] > slots.numel() else None
+    native().wkv_scan(r, k, v, wpre, w0, u, state, cu, slots, out, ws)
     return out
 
 
