@@ -12,11 +12,12 @@
 // qknorm_kv_write: RMS norm over the WHOLE q projection (all heads at once) and over the whole k projection, each
 // with its own weight vector, then q -> q_out and k, v -> their cache slots: one pass over the token's rows.
 //
-// window_attention: one wave64 per (token, head), for prompt portions and single decoded tokens alike (a sequence is
-// (cu_q[s], ctx[s]); the query at row t has position ctx - q_len + (t - cu_q)). Keys are walked in page-aligned
-// blocks of 64: lane j scores key j (q broadcast from LDS, the K row read with 16-byte loads), an online softmax
-// keeps (m, l) per wave, then lane c accumulates output channel c over the block, reading its 16 V^T values of every
-// page with 16-byte loads.
+// window_attention, row kernel: one wave64 per (token, head) (a sequence is (cu_q[s], ctx[s]); the query at row t has
+// position ctx - q_len + (t - cu_q)). Keys are walked in page-aligned blocks of 64: lane j scores key j (q broadcast
+// from LDS, the K row read with 16-byte loads), an online softmax keeps (m, l) per wave, then lane c accumulates output
+// channel c over the block, reading its 16 V^T values of every page with 16-byte loads. It serves decoded tokens, short
+// portions, fp32 activations and head sizes off the MFMA grid; bf16 prompt portions run on the query-tiled matrix-core
+// kernel further down.
 #include "gai_common.h"
 #include "gai_kernels.h"
 

@@ -11,10 +11,12 @@
 //   delta_scan        S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
 //
 // A batch is S sequences of rows [cu[s], cu[s+1]) with pool slot slots[s] (device vectors: graph-capturable); a decoded
-// token is a sequence of one row, a prompt portion a longer one, and the same kernels run both. The scans keep the
-// state in VGPRs for the whole portion: one workgroup per (head, sequence), thread (rg, j) owns rows [64 rg, 64 rg + 64)
-// of state column j, token inputs are double-buffered in LDS (two barriers per token, three when the delta rule needs
-// its read-before-write reduction across row groups), and the state is read from / written to the pool once.
+// token is a sequence of one row, a prompt portion a longer one. The scans keep the state in VGPRs for the whole
+// portion and read / write the pool once. Two shapes per recurrence:
+//   * decode steps (one row per sequence): one workgroup per (head, sequence), thread (rg, j) owns rows
+//     [64 rg, 64 rg + 64) of state column j - the state streams through coalesced, the step is state-bandwidth bound;
+//   * steps with prompt portions: the column-sliced kernels further down (one wave64 per block of state columns, no
+//     workgroup barrier in the token loop).
 #include "gai_common.h"
 #include "gai_kernels.h"
 
