@@ -63,12 +63,22 @@ class PinavikConfig:
     eos_token_ids: Tuple[int, ...] = ()
 
     def __post_init__(self):
-        self.layers = tuple(self.layers)
+        layers = []
         for i, l in enumerate(self.layers):
             if l["type"] not in MIXERS:
                 raise ValueError(f"layer {i}: unknown mixer type {l['type']!r}")
             if l.get("mlp") is not None and l["mlp"].get("kind", "dense") != "dense":
                 raise ValueError(f"layer {i}: unknown feed-forward kind {l['mlp'].get('kind')!r}")
+            m = dict(l["mixer"])  # optional keys get their neutral values: MHA, values as wide as keys, 1 / sqrt(dim)
+            if l["type"] != "wkv":
+                m.setdefault("kv_heads", m["heads"])
+                m.setdefault("vdim", m["dim"])
+                if m["heads"] % m["kv_heads"]:
+                    raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+            if l["type"] == "attention":
+                m.setdefault("scale", m["dim"] ** -0.5)
+            layers.append(dict(l, mixer=m, mlp=l.get("mlp")))
+        self.layers = tuple(layers)
         if self.loop_times and not (0 <= self.loop_start < self.loop_stop <= len(self.layers)):
             raise ValueError("loop: need 0 <= start < stop <= number of layers")
 
