@@ -77,13 +77,53 @@ void head_norm_gate(const Tensor& o, const Tensor& gate, const Tensor& nw, int64
                      y.data_ptr(), T, H, DV, (float)eps, dt, cur_stream());
 }
 
-void embed_scale_f32(const Tensor& ids, const Tensor& table, double scale, Tensor& out) {
+void embed_scale_f32(const Tensor& ids, const Tensor& table, double scale, Tensor& out,
+                     const optional<Tensor>& positions, const optional<Tensor>& pos_table) {
   const int dt = act_dt(table, "table");
   TORCH_CHECK(table.dim() == 2 && table.is_contiguous(), "embed_scale_f32: table [V, D]");
   const int T = ids.numel(), D = table.size(1);
   TORCH_CHECK(out.numel() == (int64_t)T * D, "embed_scale_f32: out shape");
+  TORCH_CHECK(positions.has_value() == pos_table.has_value(), "embed_scale_f32: positions and their table come together");
+  int P = 0;
+  if (pos_table) {
+    same_dt(*pos_table, dt, "pos_table");
+    TORCH_CHECK(pos_table->dim() == 2 && pos_table->is_contiguous() && pos_table->size(1) == D && pos_table->size(0) >= 1 &&
+                    positions->numel() >= T, "embed_scale_f32: position table [P, D], one position per token");
+    P = pos_table->size(0);
+  }
   gai_embed_scale_f32(i32(ids, "ids"), table.data_ptr(), (float)scale, f32w(out, "out"), T, D, table.size(0), dt,
-                      cur_stream());
+                      cur_stream(), positions ? i32(*positions, "positions") : nullptr,
+                      pos_table ? pos_table->data_ptr() : nullptr, P);
+}
+
+void gated_norm_add_f32(Tensor& res, const Tensor& y, const Tensor& gate, const Tensor& wpost, double eps,
+                        const optional<Tensor>& wnext, optional<Tensor> out) {
+  TORCH_CHECK(res.dim() == 2, "gated_norm_add_f32: res [T, D]");
+  float* r = f32w(res, "res");
+  const int T = res.size(0), D = res.size(1);
+  const int dty = act_dt(y, "y"), dtg = act_dt(gate, "gate");
+  TORCH_CHECK(y.size(0) == T && y.size(1) == D && gate.size(0) == T && gate.size(1) == D && wpost.numel() == D,
+              "gated_norm_add_f32: y / gate / weight shapes");
+  int dto = 0;
+  if (out) {
+    dto = act_dt(*out, "out");
+    TORCH_CHECK(out->is_contiguous() && out->numel() == (int64_t)T * D, "gated_norm_add_f32: out shape");
+  }
+  if (wnext) TORCH_CHECK(wnext->numel() == D, "gated_norm_add_f32: next norm weight size");
+  gai_gated_norm_add_f32(r, y.data_ptr(), row_stride(y, "y"), dty, gate.data_ptr(), row_stride(gate, "gate"), dtg,
+                         f32(wpost, "wpost"), wnext ? f32(*wnext, "wnext") : nullptr, out ? out->data_ptr() : nullptr,
+                         dto, T, D, (float)eps, cur_stream());
+}
+
+void gate_group_norm(const Tensor& y, const Tensor& z, const Tensor& w, int64_t groups, double eps, Tensor& out) {
+  TORCH_CHECK(y.dim() == 2, "gate_group_norm: y [T, C]");
+  const int T = y.size(0), C = y.size(1);
+  const int dt = act_dt(z, "z");
+  same_dt(out, dt, "out");
+  TORCH_CHECK(groups >= 1 && C % groups == 0 && z.size(0) == T && z.size(1) == C && w.numel() == C &&
+                  out.is_contiguous() && out.numel() == (int64_t)T * C, "gate_group_norm: shapes");
+  gai_gate_group_norm(f32(y, "y"), z.data_ptr(), row_stride(z, "z"), f32(w, "w"), out.data_ptr(), T, (int)groups,
+                      C / (int)groups, (float)eps, dt, cur_stream());
 }
 
 void check_cache(const Tensor& kc, const Tensor& vc, int dt, int G, int DK, int DV) {
@@ -113,18 +153,45 @@ void qknorm_kv_write(const Tensor& q, const Tensor& k, const Tensor& v, const Te
                       k_cache.data_ptr(), v_cache.data_ptr(), T, H, G, DK, DV, (float)eps, dt, cur_stream());
 }
 
+void headnorm_kv_write(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& wq, const Tensor& wk,
+                       const Tensor& slots, const optional<Tensor>& positions, Tensor& q_out, Tensor& k_cache,
+                       Tensor& v_cache, int64_t H, int64_t G, int64_t DK, int64_t DV, double eps, double temp_coef,
+                       int64_t temp_every) {
+  const int dt = act_dt(q, "q");
+  same_dt(k, dt, "k");
+  same_dt(v, dt, "v");
+  same_dt(q_out, dt, "q_out");
+  check_cache(k_cache, v_cache, dt, G, DK, DV);
+  const int T = q.size(0);
+  TORCH_CHECK(q.size(1) == H * DK && k.size(0) == T && k.size(1) == G * DK && v.size(0) == T && v.size(1) == G * DV,
+              "headnorm_kv_write: projection shapes");
+  TORCH_CHECK(wq.numel() == DK && wk.numel() == DK && slots.numel() >= T && q_out.is_contiguous() &&
+                  q_out.numel() == (int64_t)T * H * DK, "headnorm_kv_write: weight / slot / output shapes");
+  if (positions) TORCH_CHECK(positions->numel() >= T && temp_every >= 1, "headnorm_kv_write: one position per token");
+  gai_headnorm_kv_write(q.data_ptr(), row_stride(q, "q"), k.data_ptr(), row_stride(k, "k"), v.data_ptr(),
+                        row_stride(v, "v"), f32(wq, "wq"), f32(wk, "wk"), i32(slots, "slots"),
+                        positions ? i32(*positions, "positions") : nullptr, q_out.data_ptr(), k_cache.data_ptr(),
+                        v_cache.data_ptr(), T, H, G, DK, DV, (float)eps, (float)temp_coef, (int)temp_every, dt,
+                        cur_stream());
+}
+
 void window_attention(const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& block_tables,
                       const Tensor& cu_q, const Tensor& ctx, Tensor& out, int64_t H, int64_t G, int64_t DK, int64_t DV,
                       double scale, double softcap, int64_t window, const optional<Tensor>& r1,
-                      const optional<Tensor>& r2, const optional<Tensor>& gate) {
+                      const optional<Tensor>& r2, const optional<Tensor>& gate, const optional<Tensor>& sig_bias,
+                      bool sigmoid, double out_scale) {
   const int dt = act_dt(q, "q");
   same_dt(out, dt, "out");
   check_cache(k_cache, v_cache, dt, G, DK, DV);
-  TORCH_CHECK(q.is_contiguous() && out.is_contiguous() && q.numel() % (H * DK) == 0, "window_attention: q shape");
+  TORCH_CHECK(q.is_contiguous() && q.numel() % (H * DK) == 0, "window_attention: q shape");
   const int T = q.numel() / (H * DK);
   const int S = ctx.numel();
-  TORCH_CHECK(out.numel() == (int64_t)T * H * DV && cu_q.numel() == S + 1 && block_tables.dim() == 2 &&
+  const int ldo = row_stride(out, "out");
+  TORCH_CHECK(out.size(0) == T && out.size(1) == H * DV && cu_q.numel() == S + 1 && block_tables.dim() == 2 &&
                   block_tables.size(0) >= S, "window_attention: out / cu_q / block table shapes");
+  if (sig_bias) TORCH_CHECK(sigmoid && sig_bias->numel() == H, "window_attention: one sigmoid bias per head");
+  TORCH_CHECK(sigmoid || out_scale == 1.0, "window_attention: an output scale needs the sigmoid mode");
+  if (sigmoid) TORCH_CHECK(!gate && !r1 && softcap == 0.0, "window_attention: sigmoid mode takes no cap, distance term or gate");
   TORCH_CHECK(r1.has_value() == r2.has_value(), "window_attention: r1 and r2 come together");
   if (r1) TORCH_CHECK(r1->numel() == H && r2->numel() == H, "window_attention: one distance pair per head");
   int ldg = 0;
@@ -134,9 +201,11 @@ void window_attention(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
     TORCH_CHECK(gate->size(0) == T && gate->size(1) == H * DV, "window_attention: gate shape");
   }
   gai_window_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), i32(block_tables, "block_tables"),
-                       block_tables.size(1), i32(cu_q, "cu_q"), i32(ctx, "ctx"), S, out.data_ptr(), T, H, G, DK, DV,
+                       block_tables.size(1), i32(cu_q, "cu_q"), i32(ctx, "ctx"), S, out.data_ptr(), ldo, T, H, G, DK, DV,
                        (float)scale, (float)softcap, (int)window, r1 ? f32(*r1, "r1") : nullptr,
-                       r2 ? f32(*r2, "r2") : nullptr, gate ? gate->data_ptr() : nullptr, ldg, dt, cur_stream());
+                       r2 ? f32(*r2, "r2") : nullptr, gate ? gate->data_ptr() : nullptr, ldg,
+                       sig_bias ? f32(*sig_bias, "sig_bias") : nullptr, sigmoid ? 1 : 0, (float)out_scale, dt,
+                       cur_stream());
 }
 
 void token_shift_mix(const Tensor& h, const Tensor& mu, const Tensor& shift_state, const Tensor& cu, const Tensor& slots,
@@ -160,15 +229,62 @@ void state_tail_write(const Tensor& x, Tensor& state, const Tensor& cu, const Te
                        (int)state.size(1), dt, cur_stream());
 }
 
-void conv_silu(const Tensor& x, const Tensor& w, const Tensor& state, const Tensor& cu, const Tensor& slots, Tensor& y) {
+void conv_silu(const Tensor& x, const Tensor& w, const Tensor& state, const Tensor& cu, const Tensor& slots, Tensor& y,
+               const optional<Tensor>& bias, bool act) {
   const int dt = act_dt(x, "x");
   const int ldx = row_stride(x, "x");
   const int T = x.size(0), C = x.size(1), K = w.size(1), S = slots.numel();
   TORCH_CHECK(w.dim() == 2 && w.size(0) == C && K >= 1, "conv_silu: weight [C, taps]");
   TORCH_CHECK(state.dim() == 3 && state.size(1) == K - 1 && state.size(2) == C && cu.numel() == S + 1 &&
                   y.numel() == (int64_t)T * C, "conv_silu: state / cu / y shapes");
+  if (bias) TORCH_CHECK(bias->numel() == C, "conv_silu: one bias per channel");
   gai_conv_silu(x.data_ptr(), ldx, f32(w, "w"), f32(state, "state"), i32(cu, "cu"), i32(slots, "slots"), S,
-                f32w(y, "y"), T, C, K, dt, cur_stream());
+                f32w(y, "y"), T, C, K, dt, cur_stream(), bias ? f32(*bias, "bias") : nullptr, act ? 1 : 0);
+}
+
+void rglru_gates(const Tensor& u, const Tensor& wa_t, const Tensor& ba, const Tensor& wi_t, const Tensor& bi,
+                 const Tensor& lam, double cdecay, Tensor& a, Tensor& b) {
+  TORCH_CHECK(u.dim() == 2 && wa_t.dim() == 3 && wa_t.size(1) == wa_t.size(2), "rglru_gates: u [T, W], gates [blocks, in, out]");
+  const int T = u.size(0), W = u.size(1), NB = wa_t.size(0);
+  TORCH_CHECK(NB * wa_t.size(1) == W && wi_t.sizes() == wa_t.sizes() && ba.numel() == W && bi.numel() == W &&
+                  lam.numel() == W && a.numel() == (int64_t)T * W && b.numel() == a.numel(), "rglru_gates: shapes");
+  gai_rglru_gates(f32(u, "u"), f32(wa_t, "wa_t"), f32(ba, "ba"), f32(wi_t, "wi_t"), f32(bi, "bi"), f32(lam, "lam"),
+                  (float)cdecay, f32w(a, "a"), f32w(b, "b"), T, W, NB, cur_stream());
+}
+
+void rglru_scan(const Tensor& a, const Tensor& b, const Tensor& y, Tensor& state, const Tensor& cu, const Tensor& slots,
+                Tensor& out, bool gelu, double out_scale) {
+  TORCH_CHECK(a.dim() == 2 && state.dim() == 2, "rglru_scan: a [T, W], state [slots, W]");
+  const int T = a.size(0), W = a.size(1), S = slots.numel();
+  const int dt = act_dt(y, "y");
+  same_dt(out, dt, "out");
+  TORCH_CHECK(b.numel() == a.numel() && y.size(0) == T && y.size(1) == W && out.size(0) == T && out.size(1) == W &&
+                  state.size(1) == W && cu.numel() == S + 1, "rglru_scan: shapes");
+  gai_rglru_scan(f32(a, "a"), f32(b, "b"), y.data_ptr(), row_stride(y, "y"), f32w(state, "state"), i32(cu, "cu"),
+                 i32(slots, "slots"), S, out.data_ptr(), row_stride(out, "out"), W, gelu ? 1 : 0, (float)out_scale, dt,
+                 cur_stream());
+}
+
+void ssd_scan(const Tensor& x, const Tensor& B, const Tensor& C, const Tensor& dt, const Tensor& dt_bias,
+              const Tensor& A_log, const Tensor& D, Tensor& state, const Tensor& cu, const Tensor& slots, Tensor& out,
+              int64_t G) {
+  TORCH_CHECK(state.dim() == 4, "ssd_scan: state [slots, H, N, DV]");
+  const int H = state.size(1), N = state.size(2), DV = state.size(3), S = slots.numel();
+  auto f32row = [](const Tensor& t, const char* name) {
+    TORCH_CHECK(t.is_cuda() && t.dim() == 2 && t.scalar_type() == at::kFloat && t.stride(1) == 1, name, " must be fp32 rows");
+    return (int)t.stride(0);
+  };
+  const int ld = f32row(x, "x");
+  TORCH_CHECK(f32row(B, "B") == ld && f32row(C, "C") == ld, "ssd_scan: x / B / C must be views of one fp32 buffer");
+  const int T = x.size(0);
+  const int dtt = act_dt(dt, "dt");
+  TORCH_CHECK(x.size(1) == H * DV && B.size(0) == T && B.size(1) == G * N && C.size(0) == T && C.size(1) == G * N &&
+                  dt.size(0) == T && dt.size(1) == H && dt_bias.numel() == H && A_log.numel() == H && D.numel() == H &&
+                  cu.numel() == S + 1 && out.numel() == (int64_t)T * H * DV && G >= 1 && H % G == 0,
+              "ssd_scan: shapes");
+  gai_ssd_scan(x.data_ptr<float>(), B.data_ptr<float>(), C.data_ptr<float>(), ld, dt.data_ptr(), row_stride(dt, "dt"),
+               f32(dt_bias, "dt_bias"), f32(A_log, "A_log"), f32(D, "D"), f32w(state, "state"), i32(cu, "cu"),
+               i32(slots, "slots"), S, T, f32w(out, "out"), H, (int)G, N, DV, dtt, cur_stream());
 }
 
 void wkv_scan(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& wpre, const Tensor& w0, const Tensor& u,
@@ -241,4 +357,10 @@ void gai_bind_seq_ops(pybind11::module_& m) {
   m.def("wkv_scan", &wkv_scan);
   m.def("delta_prep", &delta_prep);
   m.def("delta_scan", &delta_scan);
+  m.def("gated_norm_add_f32", &gated_norm_add_f32);
+  m.def("gate_group_norm", &gate_group_norm);
+  m.def("headnorm_kv_write", &headnorm_kv_write);
+  m.def("rglru_gates", &rglru_gates);
+  m.def("rglru_scan", &rglru_scan);
+  m.def("ssd_scan", &ssd_scan);
 }

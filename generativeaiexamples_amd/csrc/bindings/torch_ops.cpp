@@ -377,12 +377,26 @@ void sim_topk(const Tensor& Q, const Tensor& X, const Tensor& bias, int64_t n_ro
                cur_stream());
 }
 
-void moe_route(const Tensor& logits, int64_t k, bool renorm, Tensor& ids, Tensor& w) {
+void moe_route(const Tensor& logits, int64_t k, bool renorm, Tensor& ids, Tensor& w, bool sigmoid) {
   check_f32(logits, "router logits");
   check_i32(ids, "topk ids");
   check_f32(w, "topk weights");
   gai_moe_route(logits.data_ptr<float>(), logits.size(0), logits.size(1), k, renorm ? 1 : 0, ids.data_ptr<int>(),
-                w.data_ptr<float>(), cur_stream());
+                w.data_ptr<float>(), cur_stream(), sigmoid ? 1 : 0);
+}
+
+void moe_scale_rows(const Tensor& h, const Tensor& pos, const Tensor& w, Tensor& out) {
+  check_dev(h, "h");
+  check_i32(pos, "pos");
+  check_f32(w, "w");
+  const bool f32 = h.scalar_type() == at::kFloat;
+  TORCH_CHECK((f32 || h.scalar_type() == at::kBFloat16) && out.scalar_type() == h.scalar_type(),
+              "moe_scale_rows: bf16 or fp32 rows");
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && pos.dim() == 2 && pos.is_contiguous() && w.is_contiguous() &&
+                  pos.size(0) == h.size(0) && w.numel() == pos.numel() && out.is_contiguous() &&
+                  out.numel() == pos.numel() * h.size(1), "moe_scale_rows: shapes");
+  gai_moe_scale_rows(h.data_ptr(), pos.data_ptr<int>(), w.data_ptr<float>(), out.data_ptr(), h.size(0), pos.size(1),
+                     h.size(1), f32 ? 1 : 0, cur_stream());
 }
 
 void patchify(const Tensor& img, int64_t P, const Tensor& mean, const Tensor& inv_std, Tensor& out) {
@@ -480,15 +494,25 @@ void gemm_fp8(const Tensor& A, const Tensor& B, const Tensor& sa, const Tensor& 
 }
 
 void moe_gemm(const Tensor& A, const optional<Tensor>& a_rows, const Tensor& W, Tensor& C, const Tensor& offs,
-              int64_t rows_total, bool swiglu) {
-  check_bf16(A, "A");
-  check_bf16(W, "W");
-  check_bf16(C, "C");
+              int64_t rows_total, int64_t act) {
+  const bool f32 = A.scalar_type() == at::kFloat;
+  if (f32) {
+    check_f32(A, "A");
+    check_f32(W, "W");
+    check_f32(C, "C");
+  } else {
+    check_bf16(A, "A");
+    check_bf16(W, "W");
+    check_bf16(C, "C");
+  }
   check_i32(offs, "expert offsets");
   if (a_rows) check_i32(*a_rows, "a_rows");
-  TORCH_CHECK(W.dim() == 3 && W.size(2) == A.size(-1), "moe_gemm: W must be [E, N, K]");
+  TORCH_CHECK(W.dim() == 3 && W.size(2) == A.size(-1) && W.is_contiguous() && A.is_contiguous(),
+              "moe_gemm: W must be [E, N, K]");
+  TORCH_CHECK(offs.numel() == W.size(0) + 1 && C.numel() == rows_total * (act == 1 ? W.size(1) / 2 : W.size(1)) &&
+                  (a_rows ? a_rows->numel() >= rows_total : A.size(0) >= rows_total), "moe_gemm: row / offset shapes");
   gai_moe_gemm(A.data_ptr(), a_rows ? a_rows->data_ptr<int>() : nullptr, W.data_ptr(), C.data_ptr(),
-               offs.data_ptr<int>(), W.size(0), rows_total, W.size(1), W.size(2), swiglu ? 1 : 0, cur_stream());
+               offs.data_ptr<int>(), W.size(0), rows_total, W.size(1), W.size(2), (int)act, cur_stream(), f32 ? 1 : 0);
 }
 
 void moe_dispatch(const Tensor& ids, int64_t E, Tensor& a_rows, Tensor& offs, Tensor& pos) {
@@ -507,14 +531,24 @@ void moe_dispatch(const Tensor& ids, int64_t E, Tensor& a_rows, Tensor& offs, Te
                    offs.data_ptr<int>(), pos.data_ptr<int>(), cur_stream());
 }
 
-void moe_combine(const Tensor& Y, const Tensor& pos, const Tensor& w, const optional<Tensor>& residual, Tensor& out) {
-  check_bf16(Y, "Y");
+void moe_combine(const Tensor& Y, const Tensor& pos, const optional<Tensor>& w, const optional<Tensor>& residual,
+                 Tensor& out) {
+  const bool f32 = Y.scalar_type() == at::kFloat;
+  if (f32) {
+    check_f32(Y, "Y");
+    check_f32(out, "out");
+    if (residual) check_f32(*residual, "residual");
+  } else {
+    check_bf16(Y, "Y");
+    check_bf16(out, "out");
+  }
   check_i32(pos, "pos");
-  check_f32(w, "w");
-  check_bf16(out, "out");
+  if (w) check_f32(*w, "w");
   const int T = pos.size(0), k = pos.size(1), D = out.size(-1);
-  gai_moe_combine(Y.data_ptr(), pos.data_ptr<int>(), w.data_ptr<float>(), opt_ptr(residual), out.data_ptr(), T, k, D,
-                  cur_stream());
+  TORCH_CHECK(Y.is_contiguous() && out.is_contiguous() && pos.is_contiguous() && Y.size(-1) == D &&
+                  (!w || (w->is_contiguous() && w->numel() == pos.numel())), "moe_combine: shapes");
+  gai_moe_combine(Y.data_ptr(), pos.data_ptr<int>(), w ? w->data_ptr<float>() : nullptr, opt_ptr(residual),
+                  out.data_ptr(), T, k, D, cur_stream(), f32 ? 1 : 0);
 }
 
 void embedding(const Tensor& ids, const Tensor& table, Tensor& out, int64_t vstart, int64_t vend) {
@@ -939,6 +973,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
                     (int)down, (int)offset, (int)y.numel(), (float)gain, y.data_ptr<float>(), cur_stream());
   });
   m.def("moe_route", &moe_route);
+  m.def("moe_scale_rows", &moe_scale_rows);
   m.def("moe_gemm", &moe_gemm);
   m.def("moe_combine", &moe_combine);
   m.def("moe_dispatch", &moe_dispatch);

@@ -5,7 +5,7 @@
 namespace gai {
 
 enum { EPI_NONE = 0, EPI_BIAS = 1, EPI_BIAS_GELU = 2, EPI_RESIDUAL = 3, EPI_SWIGLU = 4, EPI_BIAS_RESIDUAL = 5,
-       EPI_BIAS_RELU = 6, EPI_BIAS_QUICKGELU = 7 };
+       EPI_BIAS_RELU = 6, EPI_BIAS_QUICKGELU = 7, EPI_RELU2 = 8 };
 
 __device__ __forceinline__ float quick_gelu(float x) { return x / (1.0f + __expf(-1.702f * x)); }
 
@@ -17,6 +17,7 @@ __device__ __forceinline__ void store_out(void* C, const bf16* bias, const bf16*
   if (EPI == EPI_BIAS_GELU) v = gelu_erf(v);
   if (EPI == EPI_BIAS_RELU) v = fmaxf(v, 0.f);
   if (EPI == EPI_BIAS_QUICKGELU) v = quick_gelu(v);
+  if (EPI == EPI_RELU2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
   // residual with bf16 output = the unfused pair: bf16 projection output, then the add rounded again (the rounding of
   // the decode add+RMSNorm tails and of norm_kernel's residual add, so a fused prefill residual is bitwise theirs)
   if (EPI == EPI_RESIDUAL || EPI == EPI_BIAS_RESIDUAL) v = (OUTF32 ? v : (float)(bf16)v) + (float)R[(size_t)m * ldc + n];

@@ -137,13 +137,20 @@ void gai_ep_pack(const void* x, const int* ids, const int* offs, const int* a_pa
 void gai_ep_combine(const void* back, const int* ids, const int* pos, const int* offs, const float* w,
                     const void* residual, void* out, int T, int k, int D, int e_local, int C, hipStream_t st);
 // gemm_decode.hip: decode-sized grouped GEMM on the weight-streaming decode kernel (0 = shape not handled)
+// act: 0 none, 1 SwiGLU on the [gate16 | up16] interleave, 2 squared ReLU
 int gai_moe_gemm_dec2(const void* A, const int* a_rows, const void* W, void* C, const int* offs, int E,
-                      int rows_total, int N, int K, int swiglu, hipStream_t st);
-void gai_moe_route(const float* logits, int T, int E, int k, int renorm, int* ids, float* w, hipStream_t st);
+                      int rows_total, int N, int K, int act, hipStream_t st);
+// sigmoid: scores sigmoid(logit) per expert instead of a softmax over the experts (weights = the chosen scores)
+void gai_moe_route(const float* logits, int T, int E, int k, int renorm, int* ids, float* w, hipStream_t st,
+                   int sigmoid = 0);
+// dt: 0 bf16 (MFMA tiles when K % 64 == 0), 1 fp32 (generic grouped kernel, true fp32)
 void gai_moe_gemm(const void* A, const int* a_rows, const void* W, void* C, const int* offs, int E, int rows_total,
-                  int N, int K, int swiglu, hipStream_t st);
+                  int N, int K, int act, hipStream_t st, int dt = 0);
+// w = nullptr: plain sum of the k rows
 void gai_moe_combine(const void* Y, const int* pos, const float* w, const void* residual, void* out, int T, int k,
-                     int D, hipStream_t st);
+                     int D, hipStream_t st, int dt = 0);
+void gai_moe_scale_rows(const void* h, const int* pos, const float* w, void* out, int T, int k, int D, int dt,
+                        hipStream_t st);
 
 // misc.hip
 void gai_embedding(const int* ids, const void* table, void* out, int T, int D, int vstart, int vend, hipStream_t st);
@@ -207,22 +214,39 @@ void gai_poly_norm(const void* z, void* y, const float* coef, int T, int F, floa
 void gai_head_norm_gate(const float* o, const void* gate, int ldg, const float* nw, int nw_per_head, int act, void* y,
                         int T, int H, int DV, float eps, int dt, hipStream_t st);
 void gai_embed_scale_f32(const int* ids, const void* table, float scale, float* out, int T, int D, int V, int dt,
-                         hipStream_t st);
+                         hipStream_t st, const int* positions = nullptr, const void* pos_table = nullptr, int P = 0);
+void gai_gated_norm_add_f32(float* res, const void* y, int ldy, int dt_y, const void* gate, int ldg, int dt_gate,
+                            const float* wpost, const float* wnext, void* out, int dt_out, int T, int D, float eps,
+                            hipStream_t st);
+void gai_gate_group_norm(const float* y, const void* z, int ldz, const float* w, void* out, int T, int NG, int GS,
+                         float eps, int dt, hipStream_t st);
 // attention_window.hip
 void gai_qknorm_kv_write(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* wq,
                          const float* wk, const int* slots, void* q_out, void* k_cache, void* v_cache, int T, int H,
                          int G, int DK, int DV, float eps, int dt, hipStream_t st);
+void gai_headnorm_kv_write(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* wq,
+                           const float* wk, const int* slots, const int* positions, void* q_out, void* k_cache,
+                           void* v_cache, int T, int H, int G, int DK, int DV, float eps, float temp_coef, int temp_every,
+                           int dt, hipStream_t st);
+// sig: sigmoid weights sigmoid(score + sig_bias[h]) without normalisation over the keys, output times out_scale
 void gai_window_attention(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int maxb,
-                          const int* cu_q, const int* ctx, int S, void* out, int T, int H, int G, int DK, int DV,
+                          const int* cu_q, const int* ctx, int S, void* out, int ldo, int T, int H, int G, int DK, int DV,
                           float scale, float softcap, int window, const float* r1, const float* r2, const void* gate,
-                          int ldg, int dt, hipStream_t st);
+                          int ldg, const float* sig_bias, int sig, float out_scale, int dt, hipStream_t st);
 // recurrent.hip
 void gai_token_shift_mix(const void* h, const float* mu, int NM, const float* shift_state, const int* cu,
                          const int* slots, int S, void* out, int T, int D, int dt, hipStream_t st);
 void gai_state_tail_write(const void* x, int ldx, float* state, const int* cu, const int* slots, int S, int C, int NR,
                           int dt, hipStream_t st);
 void gai_conv_silu(const void* x, int ldx, const float* w, const float* state, const int* cu, const int* slots, int S,
-                   float* y, int T, int C, int K, int dt, hipStream_t st);
+                   float* y, int T, int C, int K, int dt, hipStream_t st, const float* bias = nullptr, int act = 1);
+void gai_rglru_gates(const float* u, const float* wa_t, const float* ba, const float* wi_t, const float* bi,
+                     const float* lam, float cdecay, float* a_out, float* b_out, int T, int W, int NB, hipStream_t st);
+void gai_rglru_scan(const float* a, const float* b, const void* y, int ldy, float* state, const int* cu,
+                    const int* slots, int S, void* out, int ldo, int W, int gelu, float scale, int dt, hipStream_t st);
+void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const void* dt, int lddt,
+                  const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu,
+                  const int* slots, int S, int T, float* out, int H, int G, int N, int DV, int dtt, hipStream_t st);
 void gai_wkv_scan(const void* r, const void* k, const void* v, int ld, const float* wpre, const float* w0,
                   const float* u, float* state, const int* cu, const int* slots, int S, int T, float* out, int H, int D,
                   int dt, float* ws, hipStream_t st);

@@ -9,6 +9,14 @@
 // K [page, G, 16, DK], V^T [page, G, DV, 16]) in bf16 or fp32; scores, softmax weights and the P.V sums are fp32.
 // Head sizes are run-time values (DK != DV allowed, DV <= 256).
 //
+// Sigmoid mode (template SIG): no softmax - a visible key weighs sigmoid(scale * (q_i . k_j) + bias_h) and the weights
+// are not normalised over the keys: o_i = out_scale * sum_j sigmoid(.) v_j. Same paging, tiling and key walk; the
+// running maximum, the rescaling of the accumulators and the final division drop out.
+//
+// headnorm_kv_write: RMS norm of every q head and every k head over its own DK channels (one weight vector of size DK
+// shared by the heads), optionally times a query temperature 1 + coef * ln(floor((p + 1) / every) + 1) of the token's
+// position p, then q -> q_out and k, v -> their cache slots; one wave64 per head.
+//
 // qknorm_kv_write: RMS norm over the WHOLE q projection (all heads at once) and over the whole k projection, each
 // with its own weight vector, then q -> q_out and k, v -> their cache slots: one pass over the token's rows.
 //
@@ -119,14 +127,57 @@ __global__ __launch_bounds__(256) void qknorm_kv_write_kernel(const TA* __restri
   }
 }
 
+template <typename TA>
+__global__ __launch_bounds__(256) void headnorm_kv_write_kernel(const TA* __restrict__ q, int ldq, const TA* __restrict__ k,
+                                                                int ldk, const TA* __restrict__ v, int ldv,
+                                                                const float* __restrict__ wq, const float* __restrict__ wk,
+                                                                const int* __restrict__ slots,
+                                                                const int* __restrict__ positions, TA* __restrict__ q_out,
+                                                                TA* __restrict__ k_cache, TA* __restrict__ v_cache, int H,
+                                                                int G, int DK, int DV, float eps, float temp_coef,
+                                                                int temp_every) {
+  const int t = blockIdx.x, wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int slot = slots[t];
+  const size_t page = slot >> 4;
+  const int off = slot & 15;
+  float temp = 1.0f;
+  if (positions) temp = 1.0f + temp_coef * logf((float)((positions[t] + 1) / temp_every + 1));
+  for (int hh = wid; hh < H + G; hh += 4) {  // q heads, then k heads: wave-uniform
+    const bool isq = hh < H;
+    const int g = isq ? hh : hh - H;
+    const TA* src = isq ? q + (size_t)t * ldq + (size_t)g * DK : k + (size_t)t * ldk + (size_t)g * DK;
+    float ss = 0.f;
+    for (int i = lane; i < DK; i += 64) {
+      const float x = (float)src[i];
+      ss += x * x;
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / DK + eps);
+    if (isq) {
+      TA* qo = q_out + ((size_t)t * H + g) * DK;
+      for (int i = lane; i < DK; i += 64) qo[i] = (TA)((float)src[i] * inv * wq[i] * temp);
+    } else {
+      TA* ko = k_cache + ((page * G + g) * 16 + off) * DK;
+      for (int i = lane; i < DK; i += 64) ko[i] = (TA)((float)src[i] * inv * wk[i]);
+    }
+  }
+  const int NV = G * DV;
+  const TA* vr = v + (size_t)t * ldv;
+  for (int i = threadIdx.x; i < NV; i += 256) {
+    const int g = i / DV, c = i - g * DV;
+    v_cache[((page * G + g) * DV + c) * 16 + off] = vr[i];
+  }
+}
+
 constexpr int kMaxVChunks = 4;  // DV <= 256
 
-template <typename TA>
+template <typename TA, bool SIG>
 __global__ __launch_bounds__(256) void window_attention_kernel(
     const TA* __restrict__ q, const TA* __restrict__ k_cache, const TA* __restrict__ v_cache,
     const int* __restrict__ block_tables, int maxb, const int* __restrict__ cu_q, const int* __restrict__ ctx, int S,
-    TA* __restrict__ out, int TH, int H, int G, int DK, int DV, float scale, float softcap, int window,
-    const float* __restrict__ r1, const float* __restrict__ r2, const TA* __restrict__ gate, int ldg, int skip_len) {
+    TA* __restrict__ out, int ldo, int TH, int H, int G, int DK, int DV, float scale, float softcap, int window,
+    const float* __restrict__ r1, const float* __restrict__ r2, const TA* __restrict__ gate, int ldg, int skip_len,
+    const float* __restrict__ sig_bias, float out_scale) {
   extern __shared__ float lds[];
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int th = blockIdx.x * 4 + wid;
@@ -148,6 +199,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
   __builtin_amdgcn_wave_barrier();
   const float b1 = r1 ? r1[h] : 0.f, b2 = r1 ? r2[h] : 0.f;
   const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+  const float pb = (SIG && sig_bias) ? sig_bias[h] : 0.f;
   const int* bt = block_tables + (size_t)s * maxb;
   float m = -INFINITY, l = 0.f, acc[kMaxVChunks];
 #pragma unroll
@@ -162,16 +214,21 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
       if (softcap > 0.f) sc = softcap * tanhf(sc * inv_cap);
       if (r1) sc -= b1 * log1pf(b2 * (float)(pos - p));
     }
-    const float m_new = fmaxf(m, wave_max(sc));
-    const float pe = valid ? expf(sc - m_new) : 0.f;
-    const float alpha = expf(m - m_new);
-    l = l * alpha + wave_sum(pe);
-    m = m_new;
+    float pe;
+    if (SIG) {
+      pe = valid ? 1.0f / (1.0f + expf(-(sc + pb))) : 0.f;
+    } else {
+      const float m_new = fmaxf(m, wave_max(sc));
+      pe = valid ? expf(sc - m_new) : 0.f;
+      const float alpha = expf(m - m_new);
+      l = l * alpha + wave_sum(pe);
+      m = m_new;
+#pragma unroll
+      for (int n = 0; n < kMaxVChunks; ++n) acc[n] *= alpha;
+    }
     __builtin_amdgcn_wave_barrier();  // the previous block's reads of ps are done
     ps[lane] = pe;
     __builtin_amdgcn_wave_barrier();
-#pragma unroll
-    for (int n = 0; n < kMaxVChunks; ++n) acc[n] *= alpha;
     for (int pg = 0; pg < 4; ++pg) {
       const int pp = kb + 16 * pg;
       if (pp > pos) break;
@@ -184,8 +241,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
       }
     }
   }
-  const float inv_l = 1.0f / l;
-  TA* o = out + (size_t)th * DV;
+  const float inv_l = SIG ? out_scale : 1.0f / l;
+  TA* o = out + (size_t)t * ldo + (size_t)h * DV;
 #pragma unroll
   for (int n = 0; n < kMaxVChunks; ++n) {
     const int c = lane + 64 * n;
@@ -228,12 +285,13 @@ __device__ __forceinline__ float tanh_fast(float y) {
   return fabsf(y) < 0.25f ? small : big;
 }
 
-template <int DK, int DV>
+template <int DK, int DV, bool SIG>
 __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
     const int* __restrict__ block_tables, int maxb, const int* __restrict__ cu_q, const int* __restrict__ ctx, int S,
-    bf16* __restrict__ out, int H, int G, float scale, float softcap, int window, const float* __restrict__ r1,
-    const float* __restrict__ r2, const bf16* __restrict__ gate, int ldg) {
+    bf16* __restrict__ out, int ldo, int H, int G, float scale, float softcap, int window, const float* __restrict__ r1,
+    const float* __restrict__ r2, const bf16* __restrict__ gate, int ldg, const float* __restrict__ sig_bias,
+    float out_scale) {
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int h = blockIdx.y * 4 + wid;
   if (h >= H) return;
@@ -264,6 +322,7 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
   float m_run = kMasked, l_run = 0.f;
   const float b1 = r1 ? r1[h] : 0.f, b2 = r1 ? r2[h] : 0.f;
   const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
+  const float pb = (SIG && sig_bias) ? sig_bias[h] : 0.f;
   for (int kb = first & ~31; kb <= last; kb += 32) {
     // ---- S^T block: rows = keys kb .. kb + 31, columns = the tile's queries
     const int kn = min(kb + qi, last);  // keys past the tile's last position: any valid row (masked below)
@@ -283,20 +342,27 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
       sc[r] = x;
       mt = fmaxf(mt, x);
     }
-    mt = max_halves(mt);
-    const float m_new = fmaxf(m_run, mt);
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * kLog2e);
-    m_run = m_new;
-    float rs = 0.f;
+    if (SIG) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float p = sc[r] > 0.5f * kMasked ? __builtin_amdgcn_exp2f((sc[r] - m_new) * kLog2e) : 0.f;
-      sc[r] = p;
-      rs += p;
+      for (int r = 0; r < 16; ++r)
+        sc[r] = sc[r] > 0.5f * kMasked
+                    ? __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-(sc[r] + pb) * kLog2e)) : 0.f;
+    } else {
+      mt = max_halves(mt);
+      const float m_new = fmaxf(m_run, mt);
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * kLog2e);
+      m_run = m_new;
+      float rs = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = sc[r] > 0.5f * kMasked ? __builtin_amdgcn_exp2f((sc[r] - m_new) * kLog2e) : 0.f;
+        sc[r] = p;
+        rs += p;
+      }
+      l_run = l_run * alpha + rs;
+#pragma unroll
+      for (int i = 0; i < DV / 32; ++i) acc_o[i] *= alpha;
     }
-    l_run = l_run * alpha + rs;
-#pragma unroll
-    for (int i = 0; i < DV / 32; ++i) acc_o[i] *= alpha;
     // ---- O^T += V^T . P^T, one 16-key page per step
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
@@ -322,8 +388,8 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
   }
   const float l = sum_halves(l_run);
   if (!valid) return;
-  const float inv_l = 1.0f / l;
-  bf16* o = out + ((size_t)t * H + h) * DV;
+  const float inv_l = SIG ? out_scale : 1.0f / l;
+  bf16* o = out + (size_t)t * ldo + (size_t)h * DV;
   const bf16* gr = gate ? gate + (size_t)t * ldg + (size_t)h * DV : nullptr;
 #pragma unroll
   for (int i = 0; i < DV / 32; ++i) {
@@ -344,13 +410,18 @@ __global__ __launch_bounds__(256) void window_attention_mfma_kernel(
 
 template <int DK, int DV>
 void launch_window_mfma(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int maxb,
-                        const int* cu_q, const int* ctx, int S, void* out, int T, int H, int G, float scale,
+                        const int* cu_q, const int* ctx, int S, void* out, int ldo, int T, int H, int G, float scale,
                         float softcap, int window, const float* r1, const float* r2, const void* gate, int ldg,
-                        hipStream_t st) {
+                        const float* sig_bias, int sig, float out_scale, hipStream_t st) {
   const dim3 grid((T + kTileQ - 1) / kTileQ + S, (H + 3) / 4);
-  window_attention_mfma_kernel<DK, DV><<<grid, 256, 0, st>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache,
-                                                             block_tables, maxb, cu_q, ctx, S, (bf16*)out, H, G, scale,
-                                                             softcap, window, r1, r2, (const bf16*)gate, ldg);
+  if (sig)
+    window_attention_mfma_kernel<DK, DV, true><<<grid, 256, 0, st>>>(
+        (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, maxb, cu_q, ctx, S, (bf16*)out, ldo, H,
+        G, scale, softcap, window, r1, r2, (const bf16*)gate, ldg, sig_bias, out_scale);
+  else
+    window_attention_mfma_kernel<DK, DV, false><<<grid, 256, 0, st>>>(
+        (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache, block_tables, maxb, cu_q, ctx, S, (bf16*)out, ldo, H,
+        G, scale, softcap, window, r1, r2, (const bf16*)gate, ldg, sig_bias, out_scale);
 }
 
 }  // namespace
@@ -370,10 +441,27 @@ void gai_qknorm_kv_write(const void* q, int ldq, const void* k, int ldk, const v
   GAI_LAUNCH_CHECK();
 }
 
+void gai_headnorm_kv_write(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, const float* wq,
+                           const float* wk, const int* slots, const int* positions, void* q_out, void* k_cache,
+                           void* v_cache, int T, int H, int G, int DK, int DV, float eps, float temp_coef, int temp_every,
+                           int dt, hipStream_t st) {
+  if (T == 0) return;
+  if (temp_every < 1) gai_launch_error(__FILE__, __LINE__, "headnorm_kv_write: temperature period must be >= 1");
+  if (dt)
+    headnorm_kv_write_kernel<float><<<T, 256, 0, st>>>((const float*)q, ldq, (const float*)k, ldk, (const float*)v, ldv,
+                                                       wq, wk, slots, positions, (float*)q_out, (float*)k_cache,
+                                                       (float*)v_cache, H, G, DK, DV, eps, temp_coef, temp_every);
+  else
+    headnorm_kv_write_kernel<bf16><<<T, 256, 0, st>>>((const bf16*)q, ldq, (const bf16*)k, ldk, (const bf16*)v, ldv, wq,
+                                                      wk, slots, positions, (bf16*)q_out, (bf16*)k_cache,
+                                                      (bf16*)v_cache, H, G, DK, DV, eps, temp_coef, temp_every);
+  GAI_LAUNCH_CHECK();
+}
+
 void gai_window_attention(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int maxb,
-                          const int* cu_q, const int* ctx, int S, void* out, int T, int H, int G, int DK, int DV,
+                          const int* cu_q, const int* ctx, int S, void* out, int ldo, int T, int H, int G, int DK, int DV,
                           float scale, float softcap, int window, const float* r1, const float* r2, const void* gate,
-                          int ldg, int dt, hipStream_t st) {
+                          int ldg, const float* sig_bias, int sig, float out_scale, int dt, hipStream_t st) {
   if (T == 0 || S == 0) return;
   if (DV > 64 * kMaxVChunks) gai_launch_error(__FILE__, __LINE__, "window_attention: value head size above 256");
   if (H % G) gai_launch_error(__FILE__, __LINE__, "window_attention: heads must be a multiple of kv heads");
@@ -382,26 +470,27 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
   // bf16 steps with prompt portions (more rows than sequences): portions of >= kMfmaMinLen rows go to the query-tiled
   // matrix-core kernel for the head sizes it is instantiated for; the rest runs below
   int skip_len = 0x7fffffff;
-  if (!dt && T > S && (!gate || ldg % 4 == 0)) {
+  if (!dt && T > S && (!gate || ldg % 4 == 0) && ldo % 4 == 0) {
 #define GAI_WIN(K_, V_)                                                                                              \
   if (DK == K_ && DV == V_) {                                                                                        \
-    launch_window_mfma<K_, V_>(q, k_cache, v_cache, block_tables, maxb, cu_q, ctx, S, out, T, H, G, scale, softcap,   \
-                               window, r1, r2, gate, ldg, st);                                                        \
+    launch_window_mfma<K_, V_>(q, k_cache, v_cache, block_tables, maxb, cu_q, ctx, S, out, ldo, T, H, G, scale,      \
+                               softcap, window, r1, r2, gate, ldg, sig_bias, sig, out_scale, st);                     \
     skip_len = kMfmaMinLen;                                                                                          \
   }
     GAI_WIN(64, 64) GAI_WIN(64, 128) GAI_WIN(128, 64) GAI_WIN(128, 128) GAI_WIN(256, 256)
 #undef GAI_WIN
     GAI_LAUNCH_CHECK();
   }
-  if (dt)
-    window_attention_kernel<float><<<grid, 256, lds, st>>>((const float*)q, (const float*)k_cache,
-                                                           (const float*)v_cache, block_tables, maxb, cu_q, ctx, S,
-                                                           (float*)out, TH, H, G, DK, DV, scale, softcap, window, r1, r2,
-                                                           (const float*)gate, ldg, skip_len);
-  else
-    window_attention_kernel<bf16><<<grid, 256, lds, st>>>((const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache,
-                                                          block_tables, maxb, cu_q, ctx, S, (bf16*)out, TH, H, G, DK,
-                                                          DV, scale, softcap, window, r1, r2, (const bf16*)gate, ldg,
-                                                          skip_len);
+#define GAI_ROW(TA, SIG_)                                                                                            \
+  window_attention_kernel<TA, SIG_><<<grid, 256, lds, st>>>((const TA*)q, (const TA*)k_cache, (const TA*)v_cache,    \
+                                                            block_tables, maxb, cu_q, ctx, S, (TA*)out, ldo, TH, H, G, \
+                                                            DK, DV, scale, softcap, window, r1, r2, (const TA*)gate,  \
+                                                            ldg, skip_len, sig_bias, out_scale)
+  if (dt) {
+    if (sig) GAI_ROW(float, true); else GAI_ROW(float, false);
+  } else {
+    if (sig) GAI_ROW(bf16, true); else GAI_ROW(bf16, false);
+  }
+#undef GAI_ROW
   GAI_LAUNCH_CHECK();
 }

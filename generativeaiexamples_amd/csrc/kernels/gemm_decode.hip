@@ -62,6 +62,7 @@ __device__ __forceinline__ float dec_act(float v, const bf16* bias, int n) {
   if (EPI == EPI_BIAS_GELU) v = gelu_erf(v);
   if (EPI == EPI_BIAS_RELU) v = fmaxf(v, 0.f);
   if (EPI == EPI_BIAS_QUICKGELU) v = quick_gelu(v);
+  if (EPI == EPI_RELU2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
   return v;
 }
 
@@ -472,7 +473,8 @@ int gai_gemm_dec2_partials(const void* A, const void* W, int M, int N, int K, fl
 // for a handful of live ones and keep one 32 KB stage in flight per CU. swiglu: W rows interleaved per 16
 // [gate16 | up16] (ops.interleave_gate_up), C = silu(gate) * up. Returns 0 when the shape does not fit.
 int gai_moe_gemm_dec2(const void* A, const int* a_rows, const void* W, void* C, const int* offs, int E,
-                      int rows_total, int N, int K, int swiglu, hipStream_t st) {
+                      int rows_total, int N, int K, int act, hipStream_t st) {
+  const int swiglu = act == 1, relu2 = act == 2;  // act: 0 none, 1 SwiGLU, 2 squared ReLU
   if (rows_total < 1 || rows_total > 64 || N % 32) return 0;
   const int ldc = swiglu ? N / 2 : N;
   const int epi = swiglu ? EPI_SWIGLU : EPI_NONE;
@@ -486,6 +488,9 @@ int gai_moe_gemm_dec2(const void* A, const int* a_rows, const void* W, void* C, 
         if constexpr (NTV >= 2)                                                                                   \
           dec2_launch<MBV, NTV, EPI_SWIGLU, false>(A, W, C, nullptr, nullptr, rows_total, N, K, ldc, st, 1,       \
                                                    nullptr, a_rows, offs, E);                                     \
+      } else if (relu2) {                                                                                         \
+        dec2_launch<MBV, NTV, EPI_RELU2, false>(A, W, C, nullptr, nullptr, rows_total, N, K, ldc, st, 1, nullptr, \
+                                                a_rows, offs, E);                                                 \
       } else {                                                                                                    \
         dec2_launch<MBV, NTV, EPI_NONE, false>(A, W, C, nullptr, nullptr, rows_total, N, K, ldc, st, 1, nullptr,  \
                                                a_rows, offs, E);                                                  \

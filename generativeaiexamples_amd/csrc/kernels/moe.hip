@@ -9,7 +9,13 @@
 //              expert by a prefix walk), so there is no host synchronisation and the launch can be
 //              captured in a HIP graph. Same 128x128x64 MFMA tile as gemm_tiled; SwiGLU epilogue for
 //              the fused w1|w3 projection.
-// moe_combine: out[t] = sum_j w[t, j] * Y[pos[t, j]] (+ residual), bf16x8 vectorised.
+//              act: SwiGLU or squared ReLU in the epilogue. fp32 operands and K off the 64 grid run on a generic
+//              LDS-tiled grouped kernel with fp32 FMA (true fp32 arithmetic).
+// moe_combine: out[t] = sum_j w[t, j] * Y[pos[t, j]] (+ residual), bf16x8 vectorised (generic kernel: fp32 rows, any
+//              width, w optional).
+// moe_route (sigmoid): every expert scored alone by sigmoid(logit); the weights are the chosen scores.
+// moe_scale_rows: expert-sorted copies of the token rows, each times its routing weight (experts whose routing weight
+//              multiplies the INPUT of a non-linear expert).
 #include "gai_common.h"
 #include "gai_kernels.h"
 
@@ -21,14 +27,15 @@ constexpr int MBM = 128, MBN = 128, MBK = 64;
 constexpr int kMTile = MBM * MBK * 2;
 
 __global__ void moe_route_kernel(const float* __restrict__ logits, int T, int E, int k, int renorm,
-                                 int* __restrict__ ids, float* __restrict__ w) {
+                                 int* __restrict__ ids, float* __restrict__ w, int sigmoid) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const float* x = logits + (size_t)t * E;
   float mx = -INFINITY;
   for (int e = 0; e < E; ++e) mx = fmaxf(mx, x[e]);
   float s = 0.f;
-  for (int e = 0; e < E; ++e) s += __expf(x[e] - mx);
+  if (!sigmoid)
+    for (int e = 0; e < E; ++e) s += __expf(x[e] - mx);
   float bv[8];
   int bi[8];
   for (int j = 0; j < k; ++j) {
@@ -36,7 +43,7 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int T, int E,
     bi[j] = 0;
   }
   for (int e = 0; e < E; ++e) {
-    const float p = __expf(x[e] - mx) / s;
+    const float p = sigmoid ? 1.0f / (1.0f + expf(-x[e])) : __expf(x[e] - mx) / s;
     if (p > bv[k - 1]) {
       int j = k - 1;
       while (j > 0 && bv[j - 1] < p) {
@@ -52,7 +59,7 @@ __global__ void moe_route_kernel(const float* __restrict__ logits, int T, int E,
   for (int j = 0; j < k; ++j) tot += bv[j];
   for (int j = 0; j < k; ++j) {
     ids[(size_t)t * k + j] = bi[j];
-    w[(size_t)t * k + j] = renorm ? bv[j] / tot : bv[j];
+    w[(size_t)t * k + j] = (renorm && !sigmoid) ? bv[j] / tot : bv[j];
   }
 }
 
@@ -60,7 +67,7 @@ __device__ __forceinline__ void glds16(const void* g, char* lds) {
   __builtin_amdgcn_global_load_lds(g, GAI_LDS(lds), 16, 0, 0);
 }
 
-template <bool SWIGLU>
+template <int ACT>  // 0 none, 1 SwiGLU, 2 squared ReLU
 __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const bf16* __restrict__ A, const int* __restrict__ a_rows,
                                                           const bf16* __restrict__ W, bf16* __restrict__ C,
                                                           const int* __restrict__ offs, int E, int N, int K) {
@@ -149,6 +156,7 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const bf16* __restrict
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
   }
+  constexpr bool SWIGLU = ACT == 1;
   const int ldc = SWIGLU ? N / 2 : N;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -166,11 +174,107 @@ __global__ __launch_bounds__(256, 2) void moe_gemm_kernel(const bf16* __restrict
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const int n = n0 + wn * 64 + 16 * j + (lane & 15);
-          if (n < N) C[(size_t)m * ldc + n] = (bf16)acc[i][j][r];
+          float v = acc[i][j][r];
+          if (ACT == 2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
+          if (n < N) C[(size_t)m * ldc + n] = (bf16)v;
         }
       }
     }
   }
+}
+
+// Generic grouped GEMM: 32 sorted rows of one expert x 64 output columns per workgroup, K walked in LDS tiles of 32,
+// fp32 FMA in ascending k. Serves fp32 models and bf16 shapes off the MFMA grid.
+template <typename TA, int ACT>
+__global__ __launch_bounds__(256) void moe_gemm_generic_kernel(const TA* __restrict__ A, const int* __restrict__ a_rows,
+                                                               const TA* __restrict__ W, TA* __restrict__ C,
+                                                               const int* __restrict__ offs, int E, int N, int K) {
+  constexpr int TM = 32, TN = 64, TK = 32;
+  __shared__ float As[TM][TK + 1];
+  __shared__ float Ws[TN][TK + 1];
+  int t = blockIdx.x, e = 0, r0 = 0, rend = 0;
+  {
+    bool found = false;
+    for (; e < E; ++e) {
+      const int cnt = offs[e + 1] - offs[e];
+      const int nt = (cnt + TM - 1) / TM;
+      if (t < nt) {
+        r0 = offs[e] + t * TM;
+        rend = offs[e + 1];
+        found = true;
+        break;
+      }
+      t -= nt;
+    }
+    if (!found) return;
+  }
+  const int n0 = blockIdx.y * TN, tid = threadIdx.x;
+  const TA* B = W + (size_t)e * N * K;
+  const int ty = tid >> 4, tx = tid & 15;  // rows 2 ty, 2 ty + 1; columns tx + 16 c
+  float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  for (int k0 = 0; k0 < K; k0 += TK) {
+    for (int x = tid; x < TM * TK; x += 256) {
+      const int r = x / TK, kk = x - r * TK, row = r0 + r;
+      float v = 0.f;
+      if (row < rend && k0 + kk < K) v = (float)A[(size_t)(a_rows ? a_rows[row] : row) * K + k0 + kk];
+      As[r][kk] = v;
+    }
+    for (int x = tid; x < TN * TK; x += 256) {
+      const int r = x / TK, kk = x - r * TK;
+      Ws[r][kk] = (n0 + r < N && k0 + kk < K) ? (float)B[(size_t)(n0 + r) * K + k0 + kk] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < TK; ++kk) {
+      const float a0 = As[2 * ty][kk], a1 = As[2 * ty + 1][kk];
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float b = Ws[tx + 16 * c][kk];
+        acc[0][c] = fmaf(a0, b, acc[0][c]);
+        acc[1][c] = fmaf(a1, b, acc[1][c]);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const int m = r0 + 2 * ty + r;
+    if (m >= rend) continue;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int n = n0 + tx + 16 * c;
+      float v = acc[r][c];
+      if (ACT == 2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
+      if (n < N) C[(size_t)m * N + n] = (TA)v;
+    }
+  }
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void moe_combine_generic_kernel(const TA* __restrict__ Y, const int* __restrict__ pos,
+                                                                  const float* __restrict__ w, const TA* residual,
+                                                                  TA* __restrict__ out, int T, int k, int D) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (long)T * D) return;
+  const int t = (int)(e / D), d = (int)(e % D);
+  float acc = 0.f;
+  for (int j = 0; j < k; ++j) {
+    const float y = (float)Y[(size_t)pos[(size_t)t * k + j] * D + d];
+    acc += w ? w[(size_t)t * k + j] * y : y;
+  }
+  if (residual) acc += (float)residual[(size_t)t * D + d];
+  out[(size_t)t * D + d] = (TA)acc;
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void moe_scale_rows_kernel(const TA* __restrict__ h, const int* __restrict__ pos,
+                                                             const float* __restrict__ w, TA* __restrict__ out, int k,
+                                                             int D) {
+  const int pair = blockIdx.x, t = pair / k;
+  const float wj = w[pair];
+  const TA* src = h + (size_t)t * D;
+  TA* dst = out + (size_t)pos[pair] * D;
+  for (int i = threadIdx.x; i < D; i += 256) dst[i] = (TA)(wj * (float)src[i]);
 }
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(const bf16* __restrict__ Y, const int* __restrict__ pos,
@@ -348,40 +452,77 @@ void gai_moe_dispatch(const int* ids, int n, int k, int E, int* a_rows, int* off
   GAI_LAUNCH_CHECK();
 }
 
-void gai_moe_route(const float* logits, int T, int E, int k, int renorm, int* ids, float* w, hipStream_t st) {
+void gai_moe_route(const float* logits, int T, int E, int k, int renorm, int* ids, float* w, hipStream_t st,
+                   int sigmoid) {
   if (T == 0) return;
-  if (k > 8) gai_launch_error(__FILE__, __LINE__, "moe_route: top-k > 8 unsupported");
-  moe_route_kernel<<<(T + 255) / 256, 256, 0, st>>>(logits, T, E, k, renorm, ids, w);
+  if (k < 1 || k > 8 || k > E) gai_launch_error(__FILE__, __LINE__, "moe_route: 1 <= top-k <= min(8, experts)");
+  moe_route_kernel<<<(T + 255) / 256, 256, 0, st>>>(logits, T, E, k, renorm, ids, w, sigmoid);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_moe_scale_rows(const void* h, const int* pos, const float* w, void* out, int T, int k, int D, int dt,
+                        hipStream_t st) {
+  if (T == 0) return;
+  if (dt)
+    moe_scale_rows_kernel<float><<<T * k, 256, 0, st>>>((const float*)h, pos, w, (float*)out, k, D);
+  else
+    moe_scale_rows_kernel<bf16><<<T * k, 256, 0, st>>>((const bf16*)h, pos, w, (bf16*)out, k, D);
   GAI_LAUNCH_CHECK();
 }
 
 void gai_moe_gemm(const void* A, const int* a_rows, const void* W, void* C, const int* offs, int E, int rows_total,
-                  int N, int K, int swiglu, hipStream_t st) {
+                  int N, int K, int act, hipStream_t st, int dt) {
   if (rows_total == 0) return;
+  if (act < 0 || act > 2) gai_launch_error(__FILE__, __LINE__, "moe_gemm: act 0 (none), 1 (SwiGLU) or 2 (squared ReLU)");
+  if (dt || K % MBK) {  // fp32 operands, or K off the MFMA tile grid: the generic grouped kernel
+    if (act == 1) gai_launch_error(__FILE__, __LINE__, "moe_gemm: SwiGLU needs bf16 operands with K % 64 == 0");
+    const dim3 grid((rows_total + 31) / 32 + E, (N + 63) / 64);
+#define GAI_MG(TA, ACT_)                                                                                        \
+  moe_gemm_generic_kernel<TA, ACT_><<<grid, 256, 0, st>>>((const TA*)A, a_rows, (const TA*)W, (TA*)C, offs, E, N, K)
+    if (dt) {
+      if (act == 2) GAI_MG(float, 2); else GAI_MG(float, 0);
+    } else {
+      if (act == 2) GAI_MG(bf16, 2); else GAI_MG(bf16, 0);
+    }
+#undef GAI_MG
+    GAI_LAUNCH_CHECK();
+    return;
+  }
   // decode steps (<= 64 expert rows in all): every expert's weights streamed once by the decode kernel
-  if (gai_moe_gemm_dec2(A, a_rows, W, C, offs, E, rows_total, N, K, swiglu, st)) return;
-  if (K % MBK) gai_launch_error(__FILE__, __LINE__, "moe_gemm: K must be a multiple of 64");
+  if (gai_moe_gemm_dec2(A, a_rows, W, C, offs, E, rows_total, N, K, act, st)) return;
   const dim3 grid((rows_total + MBM - 1) / MBM + E, (N + MBN - 1) / MBN);
   const int lds = 4 * kMTile;
   static bool once = false;
   if (!once) {
-    hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gemm_kernel<true>),
-                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-    hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gemm_kernel<false>),
-                        hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gemm_kernel<0>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gemm_kernel<1>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gemm_kernel<2>), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     once = true;
   }
-  if (swiglu) {
-    moe_gemm_kernel<true><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K);
+  if (act == 1) {
+    moe_gemm_kernel<1><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K);
+  } else if (act == 2) {
+    moe_gemm_kernel<2><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K);
   } else {
-    moe_gemm_kernel<false><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K);
+    moe_gemm_kernel<0><<<grid, 256, lds, st>>>((const bf16*)A, a_rows, (const bf16*)W, (bf16*)C, offs, E, N, K);
   }
   GAI_LAUNCH_CHECK();
 }
 
 void gai_moe_combine(const void* Y, const int* pos, const float* w, const void* residual, void* out, int T, int k,
-                     int D, hipStream_t st) {
+                     int D, hipStream_t st, int dt) {
   if (T == 0) return;
+  if (dt || D % 8 || !w) {
+    const long n = (long)T * D;
+    if (dt)
+      moe_combine_generic_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(
+          (const float*)Y, pos, w, (const float*)residual, (float*)out, T, k, D);
+    else
+      moe_combine_generic_kernel<bf16><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(
+          (const bf16*)Y, pos, w, (const bf16*)residual, (bf16*)out, T, k, D);
+    GAI_LAUNCH_CHECK();
+    return;
+  }
   const long n = (long)T * (D / 8);
   moe_combine_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>((const bf16*)Y, pos, w, (const bf16*)residual,
                                                                    (bf16*)out, T, k, D);

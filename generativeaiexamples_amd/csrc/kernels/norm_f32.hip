@@ -4,7 +4,11 @@
 //   add_rmsnorm_f32   res += mult * delta;  out = res * rsqrt(mean(res^2) + eps) * w      (w = nullptr: out = res)
 //   poly_norm         y = a N(z) + b N(z^2) + c N(z^3) + e,  N(t) = t * rsqrt(mean(t^2) + eps) over the row
 //   head_norm_gate    y = o * rsqrt(mean_head(o^2) + eps) * nw * act(gate)   (act: silu | sigmoid), one head per wave
-//   embed_scale_f32   out = table[id] * scale as fp32
+//   embed_scale_f32   out = table[id] * scale as fp32 (+ pos_table[position]: learned absolute positions)
+//   gated_norm_add    g = y * sigmoid(gate);  res += g * rsqrt(mean(g^2) + eps) * wpost;  out = rmsnorm(res) * wnext
+//                     (post-norm gated residual: the closing norm of a sublayer, the residual add and the opening norm
+//                     of the next sublayer in one pass)
+//   gate_group_norm   g = y * silu(z);  out = g * rsqrt(mean_group(g^2) + eps) * w, the row cut into equal groups
 //
 // Activations (delta, z, gate, out, y) are bf16 or fp32 (template TA); every statistic and product is fp32.
 // One wave64 per row for the row norms (D of a few thousand: the row is re-read from L2 in the second pass).
@@ -99,7 +103,8 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
 template <typename TA>
 __global__ __launch_bounds__(256) void embed_scale_f32_kernel(const int* __restrict__ ids, const TA* __restrict__ table,
                                                               float scale, float* __restrict__ out, int T, int D,
-                                                              int V) {
+                                                              int V, const int* __restrict__ positions,
+                                                              const TA* __restrict__ pos_table, int P) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= T) return;
@@ -107,7 +112,77 @@ __global__ __launch_bounds__(256) void embed_scale_f32_kernel(const int* __restr
   id = id < 0 ? 0 : (id >= V ? V - 1 : id);
   const TA* e = table + (size_t)id * D;
   float* o = out + (size_t)row * D;
-  for (int i = lane; i < D; i += 64) o[i] = (float)e[i] * scale;
+  if (pos_table) {
+    int p = positions[row];
+    p = p < 0 ? 0 : (p >= P ? P - 1 : p);
+    const TA* pe = pos_table + (size_t)p * D;
+    for (int i = lane; i < D; i += 64) o[i] = (float)e[i] * scale + (float)pe[i];
+  } else {
+    for (int i = lane; i < D; i += 64) o[i] = (float)e[i] * scale;
+  }
+}
+
+template <typename TY, typename TG, typename TA>
+__global__ __launch_bounds__(256) void gated_norm_add_kernel(float* __restrict__ res, const TY* __restrict__ y, int ldy,
+                                                             const TG* __restrict__ gate, int ldg,
+                                                             const float* __restrict__ wpost,
+                                                             const float* __restrict__ wnext, TA* __restrict__ out,
+                                                             int T, int D, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= T) return;
+  float* r = res + (size_t)row * D;
+  const TY* yr = y + (size_t)row * ldy;
+  const TG* gr = gate + (size_t)row * ldg;
+  float s = 0.f;
+  for (int i = lane; i < D; i += 64) {
+    const float g = (float)yr[i] / (1.0f + expf(-(float)gr[i]));
+    s += g * g;
+  }
+  s = wave_sum(s);
+  const float inv = 1.0f / sqrtf(s / D + eps);
+  float s2 = 0.f;
+  for (int i = lane; i < D; i += 64) {
+    const float g = (float)yr[i] / (1.0f + expf(-(float)gr[i]));
+    const float v = r[i] + g * inv * wpost[i];
+    r[i] = v;
+    s2 += v * v;
+  }
+  if (!out) return;
+  TA* o = out + (size_t)row * D;
+  if (!wnext) {
+    for (int i = lane; i < D; i += 64) o[i] = (TA)r[i];
+    return;
+  }
+  s2 = wave_sum(s2);
+  const float inv2 = 1.0f / sqrtf(s2 / D + eps);
+  for (int i = lane; i < D; i += 64) o[i] = (TA)(r[i] * inv2 * wnext[i]);
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void gate_group_norm_kernel(const float* __restrict__ y, const TA* __restrict__ z,
+                                                              int ldz, const float* __restrict__ w, TA* __restrict__ out,
+                                                              int TG, int NG, int GS, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int tg = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (tg >= TG) return;
+  const int t = tg / NG, g = tg - t * NG;
+  const float* yr = y + ((size_t)t * NG + g) * GS;
+  const TA* zr = z + (size_t)t * ldz + (size_t)g * GS;
+  float s = 0.f;
+  for (int i = lane; i < GS; i += 64) {
+    const float zv = (float)zr[i];
+    const float v = yr[i] * zv / (1.0f + expf(-zv));
+    s += v * v;
+  }
+  s = wave_sum(s);
+  const float inv = 1.0f / sqrtf(s / GS + eps);
+  const float* wr = w + (size_t)g * GS;
+  TA* o = out + ((size_t)t * NG + g) * GS;
+  for (int i = lane; i < GS; i += 64) {
+    const float zv = (float)zr[i];
+    o[i] = (TA)(yr[i] * zv / (1.0f + expf(-zv)) * inv * wr[i]);
+  }
 }
 
 }  // namespace
@@ -149,12 +224,41 @@ void gai_head_norm_gate(const float* o, const void* gate, int ldg, const float* 
 }
 
 void gai_embed_scale_f32(const int* ids, const void* table, float scale, float* out, int T, int D, int V, int dt,
-                         hipStream_t st) {
+                         hipStream_t st, const int* positions, const void* pos_table, int P) {
   if (T == 0) return;
   const int grid = (T + 3) / 4;
   if (dt)
-    embed_scale_f32_kernel<float><<<grid, 256, 0, st>>>(ids, (const float*)table, scale, out, T, D, V);
+    embed_scale_f32_kernel<float><<<grid, 256, 0, st>>>(ids, (const float*)table, scale, out, T, D, V, positions,
+                                                        (const float*)pos_table, P);
   else
-    embed_scale_f32_kernel<bf16><<<grid, 256, 0, st>>>(ids, (const bf16*)table, scale, out, T, D, V);
+    embed_scale_f32_kernel<bf16><<<grid, 256, 0, st>>>(ids, (const bf16*)table, scale, out, T, D, V, positions,
+                                                       (const bf16*)pos_table, P);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_gated_norm_add_f32(float* res, const void* y, int ldy, int dt_y, const void* gate, int ldg, int dt_gate,
+                            const float* wpost, const float* wnext, void* out, int dt_out, int T, int D, float eps,
+                            hipStream_t st) {
+  if (T == 0) return;
+  const int grid = (T + 3) / 4;
+#define GAI_GNA(TY, TG, TA)                                                                                          \
+  gated_norm_add_kernel<TY, TG, TA><<<grid, 256, 0, st>>>(res, (const TY*)y, ldy, (const TG*)gate, ldg, wpost, wnext, \
+                                                          (TA*)out, T, D, eps)
+  if (dt_y && dt_gate && (dt_out || !out)) GAI_GNA(float, float, float);
+  else if (!dt_y && !dt_gate && (!dt_out || !out)) GAI_GNA(bf16, bf16, bf16);
+  else if (!dt_y && dt_gate && (!dt_out || !out)) GAI_GNA(bf16, float, bf16);
+  else gai_launch_error(__FILE__, __LINE__, "gated_norm_add_f32: unsupported dtype combination");
+#undef GAI_GNA
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_gate_group_norm(const float* y, const void* z, int ldz, const float* w, void* out, int T, int NG, int GS,
+                         float eps, int dt, hipStream_t st) {
+  if (T == 0) return;
+  const int TG = T * NG, grid = (TG + 3) / 4;
+  if (dt)
+    gate_group_norm_kernel<float><<<grid, 256, 0, st>>>(y, (const float*)z, ldz, w, (float*)out, TG, NG, GS, eps);
+  else
+    gate_group_norm_kernel<bf16><<<grid, 256, 0, st>>>(y, (const bf16*)z, ldz, w, (bf16*)out, TG, NG, GS, eps);
   GAI_LAUNCH_CHECK();
 }

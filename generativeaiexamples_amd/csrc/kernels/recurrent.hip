@@ -1,14 +1,21 @@
 // Recurrent sequence mixers over a per-sequence fp32 state pool (slot = one live sequence):
 //
 //   token_shift_mix   m_s[t] = h[t] + (h[t-1] - h[t]) * mu_s   for NM mixes; h[-1] of a portion comes from the pool
-//   conv_silu         short causal depthwise convolution over time (last tap = current token) + SiLU; the inputs before
-//                     a portion's first token come from the pool (zeros for a fresh sequence)
+//   conv_silu         short causal depthwise convolution over time (last tap = current token) (+ bias) + SiLU (or no
+//                     activation); the inputs before a portion's first token come from the pool (zeros for a fresh
+//                     sequence)
 //   state_tail_write  keep the last NR input rows of every sequence in the pool (token shift: NR = 1; conv: taps - 1)
 //   wkv_scan          S [DK, DV] per head:  o_t = (S + diag(u) k_t v_t^T)^T r_t;  S <- diag(w_t) S + k_t v_t^T,
 //                     w_t = exp(-exp(wpre_t + w0))
 //   delta_prep        token-parallel inputs of the delta rule: unit-norm q (x DK^-1/2) and k per head, per-channel
 //                     decay exp(-exp(A_log_h) softplus(a + dt_bias)), write strength sigmoid(b)
 //   delta_scan        S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t
+//   rglru_gates       real-gated linear recurrent unit, token-parallel part: block-diagonal gates r, i = sigmoid(W u + b)
+//                     in fp32, a = exp(-c r softplus(lam)), b = sqrt(1 - a^2) i u
+//   rglru_scan        S <- a_t S + b_t per channel; o_t = scale * S_t * act(y_t)
+//   ssd_scan          state-space scan with one decay per head: S [N, DV], dt_t = softplus(dt + dt_bias),
+//                     S <- exp(-exp(A_log) dt_t) S + dt_t B_t x_t^T;  o_t = S^T C_t + D x_t  (the output reads the
+//                     UPDATED state)
 //
 // A batch is S sequences of rows [cu[s], cu[s+1]) with pool slot slots[s] (device vectors: graph-capturable); a decoded
 // token is a sequence of one row, a prompt portion a longer one. The scans keep the state in VGPRs for the whole
@@ -77,7 +84,7 @@ template <typename TA>
 __global__ __launch_bounds__(256) void conv_silu_kernel(const TA* __restrict__ x, int ldx, const float* __restrict__ w,
                                                         const float* __restrict__ state, const int* __restrict__ cu,
                                                         const int* __restrict__ slots, int S, float* __restrict__ y,
-                                                        int C, int K) {
+                                                        int C, int K, const float* __restrict__ bias, int act) {
   const int t = blockIdx.x;
   int lo = 0, hi = S;
   while (hi - lo > 1) {
@@ -93,7 +100,8 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const TA* __restrict__ x
       const float xv = src >= 0 ? (float)x[(size_t)(t - (K - 1) + i) * ldx + c] : st[(size_t)(K - 1 + src) * C + c];
       a = fmaf(xv, w[(size_t)c * K + i], a);
     }
-    y[(size_t)t * C + c] = a / (1.0f + expf(-a));
+    if (bias) a += bias[c];
+    y[(size_t)t * C + c] = act ? a / (1.0f + expf(-a)) : a;
   }
 }
 
@@ -484,6 +492,256 @@ __global__ __launch_bounds__(64) void delta_scan_cols_kernel(const float* __rest
   }
 }
 
+// ---- real-gated linear recurrent unit -----------------------------------------------------------------------------
+// Gates: one workgroup per (tile of kGT tokens, block of the block-diagonal matrices). The tile's u rows sit in LDS;
+// thread c owns output channel c of the block for all kGT tokens and walks the block's input channels: the two weight
+// reads are coalesced over the threads ([block, in, out] layout), the u reads are LDS broadcasts. All fp32 FMA: these
+// gates steer a recurrence, so they are not rounded to the matrix cores' input format.
+constexpr int kGT = 8;
+
+__device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+__global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restrict__ u, const float* __restrict__ wa_t,
+                                                          const float* __restrict__ ba, const float* __restrict__ wi_t,
+                                                          const float* __restrict__ bi, const float* __restrict__ lam,
+                                                          float cdecay, float* __restrict__ a_out,
+                                                          float* __restrict__ b_out, int T, int W, int BS) {
+  extern __shared__ float us[];  // [kGT][BS]
+  const int t0 = blockIdx.x * kGT, blk = blockIdx.y, nt = min(kGT, T - t0);
+  for (int x = threadIdx.x; x < kGT * BS; x += 256) {
+    const int tt = x / BS, k = x - tt * BS;
+    us[x] = tt < nt ? u[(size_t)(t0 + tt) * W + (size_t)blk * BS + k] : 0.f;
+  }
+  __syncthreads();
+  const float* wa = wa_t + (size_t)blk * BS * BS;
+  const float* wi = wi_t + (size_t)blk * BS * BS;
+  for (int c = threadIdx.x; c < BS; c += 256) {
+    float ar[kGT], ai[kGT];
+#pragma unroll
+    for (int tt = 0; tt < kGT; ++tt) ar[tt] = ai[tt] = 0.f;
+    for (int k = 0; k < BS; ++k) {
+      const float xa = wa[(size_t)k * BS + c], xi = wi[(size_t)k * BS + c];
+#pragma unroll
+      for (int tt = 0; tt < kGT; ++tt) {
+        const float uv = us[tt * BS + k];
+        ar[tt] = fmaf(xa, uv, ar[tt]);
+        ai[tt] = fmaf(xi, uv, ai[tt]);
+      }
+    }
+    const int ch = blk * BS + c;
+    const float sp = softplus_f(lam[ch]), rb = ba[ch], ib = bi[ch];
+#pragma unroll
+    for (int tt = 0; tt < kGT; ++tt) {
+      if (tt < nt) {
+        const float r = 1.0f / (1.0f + expf(-(ar[tt] + rb)));
+        const float ig = 1.0f / (1.0f + expf(-(ai[tt] + ib)));
+        const float la = -cdecay * r * sp;
+        const size_t o = (size_t)(t0 + tt) * W + ch;
+        a_out[o] = expf(la);
+        b_out[o] = sqrtf(-expm1f(2.0f * la)) * ig * us[tt * BS + c];
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// One thread per (sequence, channel); the loads of a step do not depend on the recurrence, so four steps are in flight.
+template <typename TA>
+__global__ __launch_bounds__(256) void rglru_scan_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                         const TA* __restrict__ y, int ldy, float* __restrict__ state,
+                                                         const int* __restrict__ cu, const int* __restrict__ slots,
+                                                         TA* __restrict__ out, int ldo, int W, int gelu, float scale) {
+  const int s = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= W) return;
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;
+  float* sp = state + (size_t)slots[s] * W + c;
+  float S = *sp;
+  int t = t0;
+  for (; t + 4 <= t1; t += 4) {
+    float av[4], bv[4], yv[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      av[x] = a[(size_t)(t + x) * W + c];
+      bv[x] = b[(size_t)(t + x) * W + c];
+      yv[x] = (float)y[(size_t)(t + x) * ldy + c];
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      S = fmaf(av[x], S, bv[x]);
+      out[(size_t)(t + x) * ldo + c] = (TA)(scale * S * (gelu ? gelu_tanh_f(yv[x]) : yv[x]));
+    }
+  }
+  for (; t < t1; ++t) {
+    S = fmaf(a[(size_t)t * W + c], S, b[(size_t)t * W + c]);
+    const float yv = (float)y[(size_t)t * ldy + c];
+    out[(size_t)t * ldo + c] = (TA)(scale * S * (gelu ? gelu_tanh_f(yv) : yv));
+  }
+  *sp = S;
+}
+
+// ---- state-space scan with a scalar decay per head ----------------------------------------------------------------
+// The two shapes of wkv_scan / delta_scan: decode steps with one workgroup per (head, sequence), prompt portions with
+// one wave64 per block of state columns.
+template <typename TA>
+__global__ __launch_bounds__(1024) void ssd_scan_kernel(const float* __restrict__ x, const float* __restrict__ Bm,
+                                                        const float* __restrict__ Cm, int ld, const TA* __restrict__ dt,
+                                                        int lddt, const float* __restrict__ dt_bias,
+                                                        const float* __restrict__ A_log, const float* __restrict__ Dskip,
+                                                        float* __restrict__ state, const int* __restrict__ cu,
+                                                        const int* __restrict__ slots, float* __restrict__ out, int H,
+                                                        int G, int N, int DV) {
+  extern __shared__ float lds[];  // buf[2][2][N] (B, C) | red[2][RG][DV]
+  const int h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
+  const int RG = (N + kRows - 1) / kRows;
+  const int j = tid % DV, rg = tid / DV;
+  const int row0 = rg * kRows, nrow = min(kRows, N - row0);
+  const int g = h / (H / G);
+  float* buf = lds;
+  float* red = buf + 4 * N;
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;
+  float* Sg = state + (((size_t)slots[s] * H + h) * N + row0) * DV + j;
+  float col[kRows];
+#pragma unroll
+  for (int i = 0; i < kRows; ++i) col[i] = i < nrow ? Sg[(size_t)i * DV] : 0.f;
+  const float negA = -expf(A_log[h]), dskip = Dskip[h], dtb = dt_bias[h];
+  for (int t = t0; t < t1; ++t) {
+    const int b = (t - t0) & 1;
+    float* bb = buf + b * 2 * N;
+    for (int i = tid; i < N; i += blockDim.x) {
+      bb[i] = Bm[(size_t)t * ld + (size_t)g * N + i];
+      bb[N + i] = Cm[(size_t)t * ld + (size_t)g * N + i];
+    }
+    const float xj = x[(size_t)t * ld + (size_t)h * DV + j];
+    const float dtv = softplus_f((float)dt[(size_t)t * lddt + h] + dtb);
+    const float dec = expf(negA * dtv), dx = dtv * xj;
+    __syncthreads();
+    float acc = 0.f;
+#pragma unroll
+    for (int i = 0; i < kRows; ++i) {
+      if (i < nrow) {
+        col[i] = fmaf(dec, col[i], bb[row0 + i] * dx);
+        acc = fmaf(col[i], bb[N + row0 + i], acc);
+      }
+    }
+    if (RG == 1) {
+      out[((size_t)t * H + h) * DV + j] = fmaf(dskip, xj, acc);
+    } else {
+      red[(b * RG + rg) * DV + j] = acc;
+      __syncthreads();
+      if (rg == 0) {
+        float o = 0.f;
+        for (int q = 0; q < RG; ++q) o += red[(b * RG + q) * DV + j];
+        out[((size_t)t * H + h) * DV + j] = fmaf(dskip, xj, o);
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < kRows; ++i)
+    if (i < nrow) Sg[(size_t)i * DV] = col[i];
+}
+
+template <typename TA, int R, int RGS>
+__global__ __launch_bounds__(64) void ssd_scan_cols_kernel(const float* __restrict__ x, const float* __restrict__ Bm,
+                                                           const float* __restrict__ Cm, int ld,
+                                                           const TA* __restrict__ dt, int lddt,
+                                                           const float* __restrict__ dt_bias,
+                                                           const float* __restrict__ A_log,
+                                                           const float* __restrict__ Dskip, float* __restrict__ state,
+                                                           const int* __restrict__ cu, const int* __restrict__ slots,
+                                                           float* __restrict__ out, int H, int G, int N, int DV) {
+  constexpr int COLS = 64 / RGS, NP = kTB * RGS * R / 64, LD = RGS * R + RGS;
+  extern __shared__ float lds[];
+  const int h = blockIdx.x, s = blockIdx.y, cb = blockIdx.z, lane = threadIdx.x;
+  const int jj = lane / RGS, rg = lane % RGS, j = cb * COLS + jj;
+  const bool on = j < DV;
+  const int row0 = rg * R, nrow = max(0, min(R, N - row0));
+  const int g = h / (H / G);
+  float* Bs = lds;
+  float* Cs = Bs + kTB * LD;
+  float* xs = Cs + kTB * LD;     // [kTB][COLS]
+  float* ds = xs + kTB * COLS;   // [2][kTB]: step size, decay
+  const int t0 = cu[s], t1 = cu[s + 1];
+  if (t1 <= t0) return;
+  for (int q = lane; q < 2 * kTB * LD; q += 64) lds[q] = 0.f;
+  float* Sg = state + (((size_t)slots[s] * H + h) * N + row0) * DV + j;
+  float col[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) col[i] = (on && i < nrow) ? Sg[(size_t)i * DV] : 0.f;
+  const float negA = -expf(A_log[h]), dskip = Dskip[h], dtb = dt_bias[h];
+  constexpr int NPART = 64 / kTB;
+  static_assert(NP * NPART >= RGS * R, "staging covers a full row");
+  const int stt = lane / NPART, spart = lane % NPART;
+  float pB[NP], pC[NP], pv[2], pdt = 0.f, pdec = 0.f;
+  auto fetch = [&](int tb) {
+    const int n = min(kTB, t1 - tb);
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      const int i = spart + NPART * q;
+      if (stt < n && i < N) {
+        const size_t o = (size_t)(tb + stt) * ld + (size_t)g * N + i;
+        pB[q] = Bm[o];
+        pC[q] = Cm[o];
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const int idx = q * 64 + lane, tt = idx / COLS, c = cb * COLS + idx % COLS;
+      pv[q] = (tt < n && c < DV) ? x[(size_t)(tb + tt) * ld + (size_t)h * DV + c] : 0.f;
+    }
+    if (lane < n) {
+      pdt = softplus_f((float)dt[(size_t)(tb + lane) * lddt + h] + dtb);
+      pdec = expf(negA * pdt);
+    }
+  };
+  fetch(t0);
+  for (int tb = t0; tb < t1; tb += kTB) {
+    const int n = min(kTB, t1 - tb);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int q = 0; q < NP; ++q) {
+      const int i = spart + NPART * q;
+      if (stt < n && i < N) {
+        const int a = stt * LD + lds_row<R>(i);
+        Bs[a] = pB[q];
+        Cs[a] = pC[q];
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      if (q * 64 + lane < kTB * COLS) xs[q * 64 + lane] = pv[q];
+    if (lane < kTB) {
+      ds[lane] = pdt;
+      ds[kTB + lane] = pdec;
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (tb + kTB < t1) fetch(tb + kTB);
+    for (int tt = 0; tt < n; ++tt) {
+      const float xj = xs[tt * COLS + jj], dec = ds[kTB + tt], dx = ds[tt] * xj;
+      const int a = tt * LD + row0 + rg;
+      float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < R; i += 2) {
+        col[i] = fmaf(dec, col[i], Bs[a + i] * dx);
+        col[i + 1] = fmaf(dec, col[i + 1], Bs[a + i + 1] * dx);
+        acc0 = fmaf(col[i], Cs[a + i], acc0);
+        acc1 = fmaf(col[i + 1], Cs[a + i + 1], acc1);
+      }
+      const float acc = rowgroup_sum<RGS>(acc0 + acc1);
+      if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * DV + j] = fmaf(dskip, xj, acc);
+    }
+  }
+  if (on) {
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+      if (i < nrow) Sg[(size_t)i * DV] = col[i];
+  }
+}
+
 }  // namespace
 
 void gai_token_shift_mix(const void* h, const float* mu, int NM, const float* shift_state, const int* cu,
@@ -509,12 +767,12 @@ void gai_state_tail_write(const void* x, int ldx, float* state, const int* cu, c
 }
 
 void gai_conv_silu(const void* x, int ldx, const float* w, const float* state, const int* cu, const int* slots, int S,
-                   float* y, int T, int C, int K, int dt, hipStream_t st) {
+                   float* y, int T, int C, int K, int dt, hipStream_t st, const float* bias, int act) {
   if (T == 0) return;
   if (dt)
-    conv_silu_kernel<float><<<T, 256, 0, st>>>((const float*)x, ldx, w, state, cu, slots, S, y, C, K);
+    conv_silu_kernel<float><<<T, 256, 0, st>>>((const float*)x, ldx, w, state, cu, slots, S, y, C, K, bias, act);
   else
-    conv_silu_kernel<bf16><<<T, 256, 0, st>>>((const bf16*)x, ldx, w, state, cu, slots, S, y, C, K);
+    conv_silu_kernel<bf16><<<T, 256, 0, st>>>((const bf16*)x, ldx, w, state, cu, slots, S, y, C, K, bias, act);
   GAI_LAUNCH_CHECK();
 }
 
@@ -593,5 +851,66 @@ void gai_delta_scan(const float* q, const float* k, const float* v, int ldv, con
   const dim3 grid(H, S);
   const size_t lds = (size_t)(6 * DK + 4 * RG * DV) * sizeof(float);
   delta_scan_kernel<<<grid, DV * RG, lds, st>>>(q, k, v, ldv, decay, beta, state, cu, slots, out, H, G, DK, DV);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_rglru_gates(const float* u, const float* wa_t, const float* ba, const float* wi_t, const float* bi,
+                     const float* lam, float cdecay, float* a_out, float* b_out, int T, int W, int NB, hipStream_t st) {
+  if (T == 0) return;
+  if (NB < 1 || W % NB) gai_launch_error(__FILE__, __LINE__, "rglru_gates: width must be a multiple of the blocks");
+  const int BS = W / NB;
+  const size_t lds = (size_t)kGT * BS * sizeof(float);
+  if (lds > 64 * 1024) gai_launch_error(__FILE__, __LINE__, "rglru_gates: block size above 2048");
+  const dim3 grid((T + kGT - 1) / kGT, NB);
+  rglru_gates_kernel<<<grid, 256, lds, st>>>(u, wa_t, ba, wi_t, bi, lam, cdecay, a_out, b_out, T, W, BS);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_rglru_scan(const float* a, const float* b, const void* y, int ldy, float* state, const int* cu,
+                    const int* slots, int S, void* out, int ldo, int W, int gelu, float scale, int dt, hipStream_t st) {
+  if (S == 0) return;
+  const dim3 grid((W + 255) / 256, S);
+  if (dt)
+    rglru_scan_kernel<float><<<grid, 256, 0, st>>>(a, b, (const float*)y, ldy, state, cu, slots, (float*)out, ldo, W,
+                                                   gelu, scale);
+  else
+    rglru_scan_kernel<bf16><<<grid, 256, 0, st>>>(a, b, (const bf16*)y, ldy, state, cu, slots, (bf16*)out, ldo, W, gelu,
+                                                  scale);
+  GAI_LAUNCH_CHECK();
+}
+
+void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const void* dt, int lddt,
+                  const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu,
+                  const int* slots, int S, int T, float* out, int H, int G, int N, int DV, int dtt, hipStream_t st) {
+  if (S == 0) return;
+  if (H % G) gai_launch_error(__FILE__, __LINE__, "ssd_scan: heads must be a multiple of groups");
+  if (N > kMaxDK) gai_launch_error(__FILE__, __LINE__, "ssd_scan: state size above 256");
+  if (T > S) {  // some sequence brings more than one row: the column-sliced scan
+#define GAI_SSD(TA, R, RGS)                                                                                          \
+  do {                                                                                                               \
+    const dim3 grid(H, S, (DV + 64 / RGS - 1) / (64 / RGS));                                                         \
+    const size_t lds = (size_t)(2 * kTB * (RGS * R + RGS) + kTB * (64 / RGS) + 2 * kTB) * sizeof(float);             \
+    ssd_scan_cols_kernel<TA, R, RGS><<<grid, 64, lds, st>>>(x, B, C, ld, (const TA*)dt, lddt, dt_bias, A_log, D,    \
+                                                            state, cu, slots, out, H, G, N, DV);                    \
+  } while (0)
+    if (dtt) {
+      if (N <= 64) GAI_SSD(float, 8, 8); else if (N <= 128) GAI_SSD(float, 8, 16); else GAI_SSD(float, 16, 16);
+    } else {
+      if (N <= 64) GAI_SSD(bf16, 8, 8); else if (N <= 128) GAI_SSD(bf16, 8, 16); else GAI_SSD(bf16, 16, 16);
+    }
+#undef GAI_SSD
+    GAI_LAUNCH_CHECK();
+    return;
+  }
+  const int RG = (N + kRows - 1) / kRows;
+  if (DV * RG > 1024) gai_launch_error(__FILE__, __LINE__, "ssd_scan: value head size times state row groups above 1024");
+  const dim3 grid(H, S);
+  const size_t lds = (size_t)(4 * N + 2 * RG * DV) * sizeof(float);
+  if (dtt)
+    ssd_scan_kernel<float><<<grid, DV * RG, lds, st>>>(x, B, C, ld, (const float*)dt, lddt, dt_bias, A_log, D, state, cu,
+                                                       slots, out, H, G, N, DV);
+  else
+    ssd_scan_kernel<bf16><<<grid, DV * RG, lds, st>>>(x, B, C, ld, (const bf16*)dt, lddt, dt_bias, A_log, D, state, cu,
+                                                      slots, out, H, G, N, DV);
   GAI_LAUNCH_CHECK();
 }

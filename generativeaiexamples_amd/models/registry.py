@@ -16,6 +16,7 @@ from .mixtral import MixtralConfig, MixtralModel
 from .mllama import MllamaConfig, MllamaModel
 from .opt import OPTConfig, OPTModel
 from .pinavik import PinavikConfig, PinavikModel
+from .ronavik import RonavikConfig, RonavikModel
 from .qwen3_next import Qwen3NextConfig, Qwen3NextModel
 
 LLM_PRESETS = {
@@ -40,6 +41,8 @@ LLM_PRESETS = {
     # hybrid of windowed attention, WKV and channel-decay delta-rule layers with a looped block (fp32 residual / state)
     "tiny-pinavik": ("tiny-pinavik", lambda: PinavikConfig.tiny()),
     "pinavik-1b": ("pinavik-1b", lambda: PinavikConfig.sized(2048, 18, 5632, 16, 128)),
+    "tiny-ronavik": ("tiny-ronavik", lambda: RonavikConfig.tiny()),
+    "ronavik-1b": ("ronavik-1b", lambda: RonavikConfig.sized(2048, 12, 1408, 16, 128, experts=8, top=2)),
     "opt-125m": ("facebook/opt-125m", lambda: OPTConfig.opt_125m()),
     "mixtral-8x7b": ("mistralai/mixtral-8x7b-instruct-v0.1", lambda: MixtralConfig.mixtral_8x7b()),
     "tiny-moe": ("tiny-moe", lambda: MixtralConfig.tiny_moe()),
@@ -79,6 +82,8 @@ def build_llm(preset: str = "llama3-8b", weights: Optional[str] = None, device=N
         arch = hf.get("model_type") or str(hf.get("architecture", "llama")).lower()
         if arch == "pinavik":
             m = PinavikModel(PinavikConfig.from_json(weights), device=device, dtype=dtype or torch.bfloat16)
+        elif arch == "ronavik":
+            m = RonavikModel(RonavikConfig.from_json(weights), device=device, dtype=dtype or torch.bfloat16)
         elif arch == "opt":
             m = OPTModel(OPTConfig.from_hf(weights), device=device)
         elif arch == "mixtral":
@@ -112,6 +117,9 @@ def build_llm(preset: str = "llama3-8b", weights: Optional[str] = None, device=N
         vocab = cfg.vocab_size
     elif isinstance(cfg, PinavikConfig):
         m = PinavikModel(cfg, device=device, dtype=dtype or torch.bfloat16).random_init(seed)
+        vocab = cfg.vocab_size
+    elif isinstance(cfg, RonavikConfig):
+        m = RonavikModel(cfg, device=device, dtype=dtype or torch.bfloat16).random_init(seed)
         vocab = cfg.vocab_size
     else:
         m = LlamaModel(cfg, device=device).random_init(seed)

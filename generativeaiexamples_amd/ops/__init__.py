@@ -826,14 +826,17 @@ def decode_advance(toks, ids, pos, ctx, slots, block_tables, n_valid):
     native().decode_advance(toks, ids, pos, ctx, slots, block_tables, n_valid, BLOCK)
 
 
-def moe_route(logits: torch.Tensor, k: int, renorm: bool = True):
-    """Router softmax + top-k -> (expert ids int32 [T,k], weights fp32 [T,k])."""
+def moe_route(logits: torch.Tensor, k: int, renorm: bool = True, score: str = "softmax"):
+    """Router scores + top-k -> (expert ids int32 [T,k], weights fp32 [T,k]). score "softmax" (weights optionally
+    renormalised over the chosen experts) or "sigmoid" (each expert scored alone; weights are the chosen scores)."""
+    if score not in ("softmax", "sigmoid"):
+        raise ValueError(f"moe_route: unknown score function {score!r}")
     if not logits.is_cuda:
-        return ref.moe_route(logits, k, renorm)
+        return ref.moe_route_sigmoid(logits, k) if score == "sigmoid" else ref.moe_route(logits, k, renorm)
     T = logits.shape[0]
     ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
     w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
-    native().moe_route(logits.float().contiguous(), k, renorm, ids, w)
+    native().moe_route(logits.float().contiguous(), k, renorm, ids, w, score == "sigmoid")
     return ids, w
 
 
@@ -949,17 +952,36 @@ def ep_combine(back, ids, pos, offs, w, residual, e_local: int, capacity: int):
     return out
 
 
-def moe_gemm(A, a_rows, W, offs, rows_total: int, swiglu: bool):
-    """Grouped expert GEMM over expert-sorted rows (A rows gathered through a_rows when given)."""
+_MOE_ACT = {None: 0, "swiglu": 1, "relu2": 2}
+
+
+def moe_gemm(A, a_rows, W, offs, rows_total: int, swiglu: bool = False, act: Optional[str] = None):
+    """Grouped expert GEMM over expert-sorted rows (A rows gathered through a_rows when given). act: None, "swiglu"
+    (W rows interleaved [gate16 | up16]) or "relu2" (squared ReLU). bf16 operands with K % 64 == 0 run on the MFMA
+    tiles; fp32 operands and other shapes on the generic grouped kernel (true fp32 arithmetic)."""
+    act = "swiglu" if swiglu else act
     if not A.is_cuda:
-        return ref.moe_gemm(A, a_rows, W, offs, rows_total, swiglu)
+        return ref.moe_gemm(A, a_rows, W, offs, rows_total, True) if act == "swiglu" else \
+            ref.moe_gemm_act(A, a_rows, W, offs, rows_total, act)
     N = W.shape[1]
-    C = torch.empty(rows_total, N // 2 if swiglu else N, dtype=A.dtype, device=A.device)
-    native().moe_gemm(A.contiguous(), a_rows, W, C, offs, rows_total, swiglu)
+    C = torch.empty(rows_total, N // 2 if act == "swiglu" else N, dtype=A.dtype, device=A.device)
+    native().moe_gemm(A.contiguous(), a_rows, W, C, offs, rows_total, _MOE_ACT[act])
     return C
 
 
+def moe_scale_rows(h, pos, w):
+    """Expert-sorted copies of the token rows, each times its routing weight (for experts whose weight multiplies
+    the INPUT): out[pos[t, j]] = w[t, j] * h[t]."""
+    if not h.is_cuda:
+        return ref.moe_scale_rows(h, pos, w)
+    T, k = pos.shape
+    out = torch.empty(T * k, h.shape[1], dtype=h.dtype, device=h.device)
+    native().moe_scale_rows(h.contiguous(), pos, w, out)
+    return out
+
+
 def moe_combine(Y, pos, w, residual=None):
+    """out[t] = sum_j w[t, j] * Y[pos[t, j]] (+ residual); w None: plain sum (the weights were applied upstream)."""
     if not Y.is_cuda:
         return ref.moe_combine(Y, pos, w, residual)
     out = torch.empty(pos.shape[0], Y.shape[1], dtype=Y.dtype, device=Y.device)
@@ -1061,6 +1083,28 @@ def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
     return y
 
 
+def gated_norm_add_f32(res: torch.Tensor, y: torch.Tensor, gate: torch.Tensor, wpost: torch.Tensor, eps: float,
+                       wnext: Optional[torch.Tensor] = None, out_dtype=None):
+    """Post-norm gated residual: fp32 ``res`` (in place) += rmsnorm(y * sigmoid(gate)) * wpost, then (out_dtype given)
+    rmsnorm(res) * wnext -- or res itself when wnext is None -- in out_dtype: the closing norm of one sublayer and the
+    opening norm of the next in one pass. y / gate may be column slices of wider rows."""
+    if not res.is_cuda:
+        return ref.gated_norm_add_f32(res, y, gate, wpost, eps, wnext, out_dtype)
+    out = torch.empty(res.shape, dtype=out_dtype, device=res.device) if out_dtype is not None else None
+    native().gated_norm_add_f32(res, y, gate, wpost, float(eps), wnext, out)
+    return out
+
+
+def gate_group_norm(y: torch.Tensor, z: torch.Tensor, w: torch.Tensor, groups: int, eps: float, out_dtype):
+    """(y * silu(z)) RMS-normalised in `groups` equal parts of the row (the gate comes BEFORE the norm), times w.
+    y fp32 [T, C]; z a column slice of the projection output."""
+    if not y.is_cuda:
+        return ref.gate_group_norm(y, z, w, groups, eps, out_dtype)
+    out = torch.empty(y.shape, dtype=out_dtype, device=y.device)
+    native().gate_group_norm(y, z, w, int(groups), float(eps), out)
+    return out
+
+
 def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, nw: torch.Tensor, act: str, eps: float, out_dtype):
     """Per-head RMS norm of fp32 o [T, H, DV], times nw ([H * DV] or shared [DV]), times silu / sigmoid of gate."""
     a = {"silu": 0, "sigmoid": 1}[act]
@@ -1072,11 +1116,15 @@ def head_norm_gate(o: torch.Tensor, gate: torch.Tensor, nw: torch.Tensor, act: s
     return y
 
 
-def embed_scale_f32(ids: torch.Tensor, table: torch.Tensor, scale: float) -> torch.Tensor:
+def embed_scale_f32(ids: torch.Tensor, table: torch.Tensor, scale: float, positions: Optional[torch.Tensor] = None,
+                    pos_table: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 rows scale * table[ids] (+ pos_table[positions]: learned absolute positions, not scaled)."""
     if not table.is_cuda:
+        if pos_table is not None:
+            return ref.embed_pos_f32(ids, table, scale, positions, pos_table)
         return ref.embed_scale_f32(ids, table, scale)
     out = torch.empty(ids.numel(), table.shape[1], dtype=torch.float32, device=table.device)
-    native().embed_scale_f32(ids, table, float(scale), out)
+    native().embed_scale_f32(ids, table, float(scale), out, positions if pos_table is not None else None, pos_table)
     return out
 
 
@@ -1099,8 +1147,39 @@ def window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H: int, G: in
                                     r1, r2, gate)
     out = torch.empty(q.shape[0], H * DV, dtype=q.dtype, device=q.device)
     native().window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, out, H, G, DK, DV, float(scale),
-                              float(softcap or 0.0), int(window or 0), r1, r2, gate)
+                              float(softcap or 0.0), int(window or 0), r1, r2, gate, None, False, 1.0)
     return out
+
+
+def sigmoid_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H: int, G: int, DK: int, DV: int, scale: float,
+                      bias=None, window: int = 0, out=None, out_scale: float = 1.0):
+    """Paged causal attention without a softmax: a visible key weighs sigmoid(scale q.k + bias_h) (bias: fp32 [H] or
+    None), weights are not normalised over the keys. window > 0 limits the visible keys to the last `window`.
+    Same kernels, paging and tiling as window_attention; output [T, H * DV] times out_scale (`out` may be a column
+    slice of a wider buffer)."""
+    if not q.is_cuda:
+        y = ref.sigmoid_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H, G, DK, DV, scale, bias, window,
+                                  out_scale)
+        return _into(out, y)
+    if out is None:
+        out = torch.empty(q.shape[0], H * DV, dtype=q.dtype, device=q.device)
+    native().window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, out, H, G, DK, DV, float(scale), 0.0,
+                              int(window or 0), None, None, None, bias, True, float(out_scale))
+    return out
+
+
+def headnorm_kv_write(q, k, v, wq, wk, slots, k_cache, v_cache, H: int, G: int, DK: int, DV: int, eps: float,
+                      positions=None, temp_coef: float = 0.0, temp_every: int = 1):
+    """RMS norm of every q head and every k head over its own DK channels (weights wq / wk of size DK, shared by the
+    heads), k and v into their cache slots; returns the normalised q [T, H * DK]. With temp_coef, the query at position
+    p is multiplied by 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1) (a length-dependent query temperature)."""
+    if not q.is_cuda:
+        return ref.headnorm_kv_write(q, k, v, wq, wk, slots, k_cache, v_cache, H, G, DK, DV, eps, positions,
+                                     temp_coef, temp_every)
+    q_out = torch.empty(q.shape[0], H * DK, dtype=q.dtype, device=q.device)
+    native().headnorm_kv_write(q, k, v, wq, wk, slots, positions if temp_coef else None, q_out, k_cache, v_cache, H, G,
+                               DK, DV, float(eps), float(temp_coef or 0.0), int(temp_every or 1))
+    return q_out
 
 
 def token_shift_mix(h, mu, shift_state, cu, slots):
@@ -1119,13 +1198,54 @@ def state_tail_write(x, state, cu, slots) -> None:
     native().state_tail_write(x, state, cu, slots)
 
 
-def conv_silu(x, w, state, cu, slots):
-    """Causal depthwise conv over time (w [C, taps], last tap = current row) + SiLU -> fp32 [T, C]."""
+def conv_silu(x, w, state, cu, slots, bias=None, act: bool = True):
+    """Causal depthwise conv over time (w [C, taps], last tap = current row) (+ bias) + SiLU (act=False: none)
+    -> fp32 [T, C]."""
     if not x.is_cuda:
-        return ref.conv_silu(x, w, state, cu, slots)
+        if bias is None and act:
+            return ref.conv_silu(x, w, state, cu, slots)
+        return ref.conv_bias_act(x, w, state, cu, slots, bias, act)
     y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
-    native().conv_silu(x, w, state, cu, slots, y)
+    native().conv_silu(x, w, state, cu, slots, y, bias, bool(act))
     return y
+
+
+def rglru_gates(u, wa_t, ba, wi_t, bi, lam, c: float = 8.0):
+    """Gates of a real-gated linear recurrent unit, all fp32: u [T, W] split into nb blocks; r = sigmoid(Wa_b u_b + ba),
+    i = sigmoid(Wi_b u_b + bi) (wa_t / wi_t: [nb, in, out], the block matrices transposed); returns
+    (a, b) = (exp(-c r softplus(lam)), sqrt(1 - a^2) i u), the coefficients of S_t = a_t S_(t-1) + b_t."""
+    if not u.is_cuda:
+        return ref.rglru_gates(u, wa_t, ba, wi_t, bi, lam, c)
+    a = torch.empty(u.shape, dtype=torch.float32, device=u.device)
+    b = torch.empty_like(a)
+    native().rglru_gates(u, wa_t, ba, wi_t, bi, lam, float(c), a, b)
+    return a, b
+
+
+def rglru_scan(a, b, y, state, cu, slots, out_dtype, act: Optional[str] = None, out=None, out_scale: float = 1.0):
+    """Per-channel linear recurrence S_t = a_t S_(t-1) + b_t (state [slots, W] fp32, in place) -> out_scale * S_t *
+    act(y_t) [T, W] (act None or "gelu_tanh", applied in fp32; y and `out` may be column slices of wider rows)."""
+    if act not in (None, "gelu_tanh"):
+        raise ValueError(f"rglru_scan: unknown activation {act!r}")
+    if not a.is_cuda:
+        return _into(out, ref.rglru_scan(a, b, y, state, cu, slots, out_dtype, act, out_scale))
+    if out is None:
+        out = torch.empty(a.shape, dtype=out_dtype, device=a.device)
+    native().rglru_scan(a, b, y, state, cu, slots, out, act == "gelu_tanh", float(out_scale))
+    return out
+
+
+def ssd_scan(x, B, C, dt, dt_bias, A_log, D, state, cu, slots, G: int):
+    """State-space scan, one decay per head: S_t = exp(-exp(A_log_h) dt_t) S_(t-1) + dt_t B_t x_t^T,
+    y_t = S_t^T C_t + D_h x_t with dt_t = softplus(dt + dt_bias). x [T, H * DV], B / C [T, G * N] fp32 (column
+    slices of the convolution output), dt [T, H] a slice of the projection; state [slots, H, N, DV] in place
+    -> fp32 [T, H, DV]."""
+    if not x.is_cuda:
+        return ref.ssd_scan(x, B, C, dt, dt_bias, A_log, D, state, cu, slots, G)
+    H, DV = state.shape[1], state.shape[3]
+    out = torch.empty(x.shape[0], H, DV, dtype=torch.float32, device=x.device)
+    native().ssd_scan(x, B, C, dt, dt_bias, A_log, D, state, cu, slots, out, G)
+    return out
 
 
 def wkv_scan(r, k, v, wpre, w0, u, state, cu, slots):

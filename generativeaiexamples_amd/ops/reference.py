@@ -275,7 +275,8 @@ def moe_gemm(A, a_rows, W, offs, rows_total, swiglu):
 
 
 def moe_combine(Y, pos, w, residual=None):
-    y = (Y[pos.long()].float() * w.float()[..., None]).sum(1)
+    y = Y[pos.long()].float()
+    y = (y * w.float()[..., None]).sum(1) if w is not None else y.sum(1)
     if residual is not None:
         y = y + residual.float()
     return y.to(Y.dtype)
@@ -598,3 +599,153 @@ def delta_scan(q, k, v, decay, beta, state, cu, slots, G):
         if e > b:
             state[s] = S
     return out
+
+
+# ---------------------------------------------------------------------------------------------
+# post-norm gated residual, per-head q/k norm with a query temperature, sigmoid attention, gated linear recurrence,
+# state-space scan, sigmoid router with input-side expert weights
+# ---------------------------------------------------------------------------------------------
+def embed_pos_f32(ids, table, scale, positions, pos_table):
+    x = embed_scale_f32(ids, table, scale)
+    return x + pos_table[positions.long().clamp(0, pos_table.shape[0] - 1)].float()
+
+
+def gated_norm_add_f32(res, y, gate, wpost, eps, wnext, out_dtype):
+    """res (fp32, in place) += rmsnorm(y * sigmoid(gate)) * wpost; returns rmsnorm(res) * wnext (wnext None: res) as
+    out_dtype, or None when out_dtype is None."""
+    g = y.float() * torch.sigmoid(gate.float())
+    res.add_(g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps) * wpost.float())
+    return add_rmsnorm_f32(res, None, 1.0, wnext, eps, out_dtype)
+
+
+def headnorm_kv_write(q, k, v, wq, wk, slots, k_cache, v_cache, H, G, DK, DV, eps, positions, temp_coef, temp_every):
+    T = q.shape[0]
+    n = lambda t, w: t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w.float()  # noqa: E731
+    qn = n(q.float().reshape(T, H, DK), wq)
+    if temp_coef:
+        p = positions[:T].long()
+        qn = qn * (1.0 + float(temp_coef) * torch.log(((p + 1) // int(temp_every) + 1).float()))[:, None, None]
+    kn = n(k.float().reshape(T, G, DK), wk).to(k_cache.dtype)
+    s = slots[:T].long()
+    k_cache[s // BLOCK, :, s % BLOCK] = kn
+    v_cache[s // BLOCK, :, :, s % BLOCK] = v.reshape(T, G, DV).to(v_cache.dtype)
+    return qn.reshape(T, H * DK).to(q.dtype)
+
+
+def sigmoid_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H, G, DK, DV, scale, bias, window, out_scale=1.0):
+    """o_i = sum_j sigmoid(scale q_i . k_j + bias_h) v_j over the visible keys (no normalisation over keys)."""
+    T = q.numel() // (H * DK)
+    q3 = q.float().view(T, H, DK)
+    out = torch.zeros(T, H, DV)
+    cu = [int(x) for x in cu_q.tolist()]
+    for s, n in enumerate(ctx.tolist()):
+        b, e = cu[s], cu[s + 1]
+        if e <= b:
+            continue
+        n = int(n)
+        pages = block_tables[s, : (n + BLOCK - 1) // BLOCK].long()
+        K = k_cache[pages].float().permute(1, 0, 2, 3).reshape(G, -1, DK)[:, :n]
+        V = v_cache[pages].float().permute(1, 0, 3, 2).reshape(G, -1, DV)[:, :n]
+        pos = torch.arange(n - (e - b), n)
+        dist = pos[:, None] - torch.arange(n)[None, :]
+        vis = (dist >= 0) & ((dist < window) if window > 0 else True)
+        for h in range(H):
+            sc = (q3[b:e, h] @ K[h // (H // G)].t()) * scale + (float(bias[h]) if bias is not None else 0.0)
+            out[b:e, h] = (torch.sigmoid(sc) * vis) @ V[h // (H // G)]
+    return (out.reshape(T, H * DV) * float(out_scale)).to(q.dtype)
+
+
+def conv_bias_act(x, w, state, cu, slots, bias, act):
+    K = w.shape[1]
+    y = torch.empty(x.shape, dtype=torch.float32)
+    for b, e, s in _seqs(cu, slots):
+        if e > b:
+            xs = torch.cat([state[s], x[b:e].float()])
+            y[b:e] = (xs.unfold(0, K, 1) * w.float()).sum(-1)
+    if bias is not None:
+        y = y + bias.float()
+    return F.silu(y) if act else y
+
+
+def rglru_gates(u, wa_t, ba, wi_t, bi, lam, c):
+    """Block-diagonal gates of a real-gated linear recurrent unit. u [T, W] fp32; wa_t / wi_t [nb, in, out];
+    returns (a, b): a = exp(-c r softplus(lam)), b = sqrt(1 - a^2) i u with r, i = sigmoid(block(u) + bias)."""
+    T, W = u.shape
+    nb, bs = wa_t.shape[0], wa_t.shape[1]
+    ub = u.float().reshape(T, nb, bs).transpose(0, 1)                      # [nb, T, bs]
+    r = torch.sigmoid(torch.bmm(ub, wa_t.float()).transpose(0, 1).reshape(T, W) + ba.float().reshape(-1))
+    i = torch.sigmoid(torch.bmm(ub, wi_t.float()).transpose(0, 1).reshape(T, W) + bi.float().reshape(-1))
+    a = torch.exp(-float(c) * r * F.softplus(lam.float()))
+    return a, torch.sqrt(1.0 - a * a) * i * u.float()
+
+
+def rglru_scan(a, b, y, state, cu, slots, out_dtype, act=None, out_scale=1.0):
+    """S_t = a_t S_(t-1) + b_t per channel; returns S_t * y_t. state [slots, W] fp32 in place."""
+    out = torch.empty(a.shape, dtype=torch.float32)
+    for lo, hi, s in _seqs(cu, slots):
+        S = state[s]
+        for t in range(lo, hi):
+            S = a[t] * S + b[t]
+            out[t] = S
+        if hi > lo:
+            state[s] = S
+    yy = F.gelu(y.float(), approximate="tanh") if act == "gelu_tanh" else y.float()
+    return (out * yy * float(out_scale)).to(out_dtype)
+
+
+def ssd_scan(x, B, C, dt, dt_bias, A_log, D, state, cu, slots, G):
+    """State-space scan with one decay per head: S_t = exp(-exp(A_log) dt_t) S_(t-1) + dt_t B_t x_t^T,
+    y_t = S_t^T C_t + D x_t; dt_t = softplus(dt + dt_bias). state [slots, H, N, DV] fp32 in place."""
+    H, N, DV = state.shape[1:]
+    T = x.shape[0]
+    rep = H // G
+    x3 = x.float().reshape(T, H, DV)
+    B3 = B.float().reshape(T, G, N).repeat_interleave(rep, 1)
+    C3 = C.float().reshape(T, G, N).repeat_interleave(rep, 1)
+    dts = F.softplus(dt.float() + dt_bias.float().reshape(1, -1))          # [T, H]
+    dec = torch.exp(-torch.exp(A_log.float())[None] * dts)
+    out = torch.empty(T, H, DV)
+    for lo, hi, s in _seqs(cu, slots):
+        S = state[s]
+        for t in range(lo, hi):
+            S = dec[t][:, None, None] * S + (dts[t][:, None] * B3[t])[:, :, None] * x3[t][:, None, :]
+            out[t] = torch.einsum("hnv,hn->hv", S, C3[t]) + D.float()[:, None] * x3[t]
+        if hi > lo:
+            state[s] = S
+    return out
+
+
+def gate_group_norm(y, z, w, groups, eps, out_dtype):
+    """(y * silu(z)) RMS-normalised in `groups` equal parts of the last dim, times w."""
+    T, C = y.shape
+    g = (y.float() * F.silu(z.float())).reshape(T, groups, C // groups)
+    g = g * torch.rsqrt(g.pow(2).mean(-1, keepdim=True) + eps)
+    return (g.reshape(T, C) * w.float()).to(out_dtype)
+
+
+def moe_route_sigmoid(logits, k):
+    s = torch.sigmoid(logits.float())
+    w, ids = torch.topk(s, k, dim=-1)
+    return ids.int(), w
+
+
+def moe_scale_rows(h, pos, w):
+    """Expert-sorted copies of the token rows, each times its routing weight: out[pos[t, j]] = w[t, j] * h[t]."""
+    T, k = pos.shape
+    out = torch.empty(T * k, h.shape[1], dtype=h.dtype)
+    out[pos.reshape(-1).long()] = (h.float()[:, None, :] * w.float()[:, :, None]).reshape(T * k, -1).to(h.dtype)
+    return out
+
+
+def moe_gemm_act(A, a_rows, W, offs, rows_total, act):
+    E, N, K = W.shape
+    C = torch.empty(rows_total, N, dtype=A.dtype)
+    o = offs.tolist()
+    for e in range(E):
+        if o[e + 1] > o[e]:
+            rows = A[a_rows[o[e]:o[e + 1]].long()] if a_rows is not None else A[o[e]:o[e + 1]]
+            y = rows.float() @ W[e].float().t()
+            if act == "relu2":
+                y = torch.relu(y) ** 2
+            C[o[e]:o[e + 1]] = y.to(A.dtype)
+    return C
