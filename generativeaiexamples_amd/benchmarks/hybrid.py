@@ -1,7 +1,9 @@
 """Prefill and decode throughput of the hybrid decoders at layer sizes of real models (random weights), side by side:
-Pinavik (windowed attention + WKV + channel-decay delta rule, fp32 residual / state) and the framework's closest
-existing model, Qwen3-Next (gated full attention + gated DeltaNet), built with dense MLPs at the same width, depth,
-head geometry and feed-forward size. `bench.py --hybrid` runs it; the default workload of bench.py is untouched.
+Ronavik (sigmoid attention beside a gated linear recurrence, state-space scan layers, sigmoid-routed experts, fp32
+post-norm residual / state), Pinavik (windowed attention + WKV + channel-decay delta rule, fp32 residual / state) and
+Qwen3-Next (gated full attention + gated DeltaNet), built at the same width, depth, head geometry and active
+feed-forward size (Ronavik: 8 experts of half the dense size, 2 per token; the others dense). `bench.py --hybrid` runs
+it; the default workload of bench.py is untouched.
 
 Both models run through the serving engine (native scheduler, paged KV, state slots, decode graphs):
   * prefill: one prompt of T tokens in one step -> tokens / s;
@@ -22,9 +24,9 @@ SIZES = {  # name: (width, layers, ff, heads, head_dim)
 
 def add_args(ap):
     ap.add_argument("--hybrid", action="store_true",
-                    help="prefill / decode throughput of Pinavik beside Qwen3-Next at equal layer sizes (one GPU)")
+                    help="prefill / decode throughput of Ronavik, Pinavik and Qwen3-Next at equal layer sizes (one GPU)")
     ap.add_argument("--hybrid-sizes", default="1k,2k", help="comma list of " + ",".join(SIZES))
-    ap.add_argument("--hybrid-models", default="pinavik,qwen3-next")
+    ap.add_argument("--hybrid-models", default="ronavik,pinavik,qwen3-next")
     ap.add_argument("--hybrid-prefill", default="2048,8192", help="prompt lengths of the prefill measurement")
     ap.add_argument("--hybrid-decode", default="1,16,64", help="batch sizes of the decode measurement")
     ap.add_argument("--hybrid-context", type=int, default=1024)
@@ -33,6 +35,11 @@ def add_args(ap):
 
 def build(model: str, size: str, window: int, device):
     W, L, F, H, hd = SIZES[size]
+    if model == "ronavik":
+        from ..models.ronavik import RonavikConfig, RonavikModel
+
+        cfg = RonavikConfig.sized(W, L, F // 2, H, hd, experts=8, top=2, max_position=16384)
+        return RonavikModel(cfg, device=device).random_init(0)
     if model == "pinavik":
         from ..models.pinavik import PinavikConfig, PinavikModel
 
@@ -113,8 +120,8 @@ def run(args) -> dict:
     for size in args.hybrid_sizes.split(","):
         for name in args.hybrid_models.split(","):
             model = build(name, size, args.hybrid_window, dev)
-            r = measure(model, [int(x) for x in args.hybrid_prefill.split(",")],
-                        [int(x) for x in args.hybrid_decode.split(",")], args.hybrid_context,
+            r = measure(model, [int(x) for x in args.hybrid_prefill.split(",") if x],
+                        [int(x) for x in args.hybrid_decode.split(",") if x], args.hybrid_context,
                         max(1, args.steps), max(1, args.warmup))
             r["params_m"] = round(model.num_params() / 1e6, 1)
             res[f"{name}-{size}"] = r

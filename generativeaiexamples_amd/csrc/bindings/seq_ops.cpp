@@ -252,17 +252,25 @@ void rglru_gates(const Tensor& u, const Tensor& wa_t, const Tensor& ba, const Te
                   (float)cdecay, f32w(a, "a"), f32w(b, "b"), T, W, NB, cur_stream());
 }
 
+int64_t rglru_scan_ws_floats(int64_t T, int64_t S, int64_t W) { return 3 * (int64_t)gai_rglru_scan_chunks(T, S) * W; }
+
 void rglru_scan(const Tensor& a, const Tensor& b, const Tensor& y, Tensor& state, const Tensor& cu, const Tensor& slots,
-                Tensor& out, bool gelu, double out_scale) {
+                Tensor& out, bool gelu, double out_scale, const optional<Tensor>& ws) {
   TORCH_CHECK(a.dim() == 2 && state.dim() == 2, "rglru_scan: a [T, W], state [slots, W]");
   const int T = a.size(0), W = a.size(1), S = slots.numel();
   const int dt = act_dt(y, "y");
   same_dt(out, dt, "out");
   TORCH_CHECK(b.numel() == a.numel() && y.size(0) == T && y.size(1) == W && out.size(0) == T && out.size(1) == W &&
                   state.size(1) == W && cu.numel() == S + 1, "rglru_scan: shapes");
+  float* wsp = nullptr;
+  if (ws) {
+    TORCH_CHECK(ws->is_cuda() && ws->scalar_type() == at::kFloat && ws->is_contiguous() &&
+                    ws->numel() >= rglru_scan_ws_floats(T, S, W), "rglru_scan: workspace too small");
+    wsp = ws->data_ptr<float>();
+  }
   gai_rglru_scan(f32(a, "a"), f32(b, "b"), y.data_ptr(), row_stride(y, "y"), f32w(state, "state"), i32(cu, "cu"),
-                 i32(slots, "slots"), S, out.data_ptr(), row_stride(out, "out"), W, gelu ? 1 : 0, (float)out_scale, dt,
-                 cur_stream());
+                 i32(slots, "slots"), S, T, out.data_ptr(), row_stride(out, "out"), W, gelu ? 1 : 0, (float)out_scale,
+                 dt, wsp, cur_stream());
 }
 
 void ssd_scan(const Tensor& x, const Tensor& B, const Tensor& C, const Tensor& dt, const Tensor& dt_bias,
@@ -362,5 +370,6 @@ void gai_bind_seq_ops(pybind11::module_& m) {
   m.def("headnorm_kv_write", &headnorm_kv_write);
   m.def("rglru_gates", &rglru_gates);
   m.def("rglru_scan", &rglru_scan);
+  m.def("rglru_scan_ws_floats", &rglru_scan_ws_floats);
   m.def("ssd_scan", &ssd_scan);
 }

@@ -509,7 +509,7 @@ void moe_gemm(const Tensor& A, const optional<Tensor>& a_rows, const Tensor& W, 
   if (a_rows) check_i32(*a_rows, "a_rows");
   TORCH_CHECK(W.dim() == 3 && W.size(2) == A.size(-1) && W.is_contiguous() && A.is_contiguous(),
               "moe_gemm: W must be [E, N, K]");
-  TORCH_CHECK(offs.numel() == W.size(0) + 1 && C.numel() == rows_total * (act == 1 ? W.size(1) / 2 : W.size(1)) &&
+  TORCH_CHECK(offs.numel() >= W.size(0) + 1 && C.numel() == rows_total * (act == 1 ? W.size(1) / 2 : W.size(1)) &&
                   (a_rows ? a_rows->numel() >= rows_total : A.size(0) >= rows_total), "moe_gemm: row / offset shapes");
   gai_moe_gemm(A.data_ptr(), a_rows ? a_rows->data_ptr<int>() : nullptr, W.data_ptr(), C.data_ptr(),
                offs.data_ptr<int>(), W.size(0), rows_total, W.size(1), W.size(2), (int)act, cur_stream(), f32 ? 1 : 0);

@@ -242,8 +242,11 @@ void gai_conv_silu(const void* x, int ldx, const float* w, const float* state, c
                    float* y, int T, int C, int K, int dt, hipStream_t st, const float* bias = nullptr, int act = 1);
 void gai_rglru_gates(const float* u, const float* wa_t, const float* ba, const float* wi_t, const float* bi,
                      const float* lam, float cdecay, float* a_out, float* b_out, int T, int W, int NB, hipStream_t st);
+// ws (optional, fp32 [3][gai_rglru_scan_chunks(T, S)][W]): steps with prompt portions run the chunk-parallel scan
+int gai_rglru_scan_chunks(int T, int S);
 void gai_rglru_scan(const float* a, const float* b, const void* y, int ldy, float* state, const int* cu,
-                    const int* slots, int S, void* out, int ldo, int W, int gelu, float scale, int dt, hipStream_t st);
+                    const int* slots, int S, int T, void* out, int ldo, int W, int gelu, float scale, int dt, float* ws,
+                    hipStream_t st);
 void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const void* dt, int lddt,
                   const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu,
                   const int* slots, int S, int T, float* out, int H, int G, int N, int DV, int dtt, hipStream_t st);

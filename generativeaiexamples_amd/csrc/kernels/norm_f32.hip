@@ -159,6 +159,108 @@ __global__ __launch_bounds__(256) void gated_norm_add_kernel(float* __restrict__
   for (int i = lane; i < D; i += 64) o[i] = (TA)(r[i] * inv2 * wnext[i]);
 }
 
+// Few rows (decode steps): one workgroup per row instead of one wave, the gated values kept in registers between the
+// passes (rows up to 256 * kWideRegs wide; wider rows recompute them).
+constexpr int kWideRegs = 16;
+
+template <typename TY, typename TG, typename TA>
+__global__ __launch_bounds__(256) void gated_norm_add_wide_kernel(float* __restrict__ res, const TY* __restrict__ y,
+                                                                  int ldy, const TG* __restrict__ gate, int ldg,
+                                                                  const float* __restrict__ wpost,
+                                                                  const float* __restrict__ wnext, TA* __restrict__ out,
+                                                                  int D, float eps) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  float* r = res + (size_t)row * D;
+  const TY* yr = y + (size_t)row * ldy;
+  const TG* gr = gate + (size_t)row * ldg;
+  float g[kWideRegs];
+  float s = 0.f;
+#pragma unroll
+  for (int q = 0; q < kWideRegs; ++q) {
+    const int i = tid + 256 * q;
+    g[q] = i < D ? (float)yr[i] / (1.0f + expf(-(float)gr[i])) : 0.f;
+    s += g[q] * g[q];
+  }
+  for (int i = tid + 256 * kWideRegs; i < D; i += 256) {
+    const float v = (float)yr[i] / (1.0f + expf(-(float)gr[i]));
+    s += v * v;
+  }
+  s = block_sum(s, scratch);
+  const float inv = 1.0f / sqrtf(s / D + eps);
+  float s2 = 0.f;
+#pragma unroll
+  for (int q = 0; q < kWideRegs; ++q) {
+    const int i = tid + 256 * q;
+    if (i < D) {
+      g[q] = r[i] + g[q] * inv * wpost[i];
+      r[i] = g[q];
+      s2 += g[q] * g[q];
+    }
+  }
+  for (int i = tid + 256 * kWideRegs; i < D; i += 256) {
+    const float v = r[i] + (float)yr[i] / (1.0f + expf(-(float)gr[i])) * inv * wpost[i];
+    r[i] = v;
+    s2 += v * v;
+  }
+  if (!out) return;
+  TA* o = out + (size_t)row * D;
+  if (!wnext) {
+    for (int i = tid; i < D; i += 256) o[i] = (TA)r[i];
+    return;
+  }
+  s2 = block_sum(s2, scratch);
+  const float inv2 = 1.0f / sqrtf(s2 / D + eps);
+#pragma unroll
+  for (int q = 0; q < kWideRegs; ++q) {
+    const int i = tid + 256 * q;
+    if (i < D) o[i] = (TA)(g[q] * inv2 * wnext[i]);
+  }
+  for (int i = tid + 256 * kWideRegs; i < D; i += 256) o[i] = (TA)(r[i] * inv2 * wnext[i]);
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void gate_group_norm_wide_kernel(const float* __restrict__ y, const TA* __restrict__ z,
+                                                                   int ldz, const float* __restrict__ w,
+                                                                   TA* __restrict__ out, int NG, int GS, float eps) {
+  __shared__ float scratch[16];
+  const int tg = blockIdx.x, tid = threadIdx.x;
+  const int t = tg / NG, g = tg - t * NG;
+  const float* yr = y + ((size_t)t * NG + g) * GS;
+  const TA* zr = z + (size_t)t * ldz + (size_t)g * GS;
+  float v[kWideRegs];
+  float s = 0.f;
+#pragma unroll
+  for (int q = 0; q < kWideRegs; ++q) {
+    const int i = tid + 256 * q;
+    float x = 0.f;
+    if (i < GS) {
+      const float zv = (float)zr[i];
+      x = yr[i] * zv / (1.0f + expf(-zv));
+    }
+    v[q] = x;
+    s += x * x;
+  }
+  for (int i = tid + 256 * kWideRegs; i < GS; i += 256) {
+    const float zv = (float)zr[i];
+    const float x = yr[i] * zv / (1.0f + expf(-zv));
+    s += x * x;
+  }
+  s = block_sum(s, scratch);
+  const float inv = 1.0f / sqrtf(s / GS + eps);
+  const float* wr = w + (size_t)g * GS;
+  TA* o = out + ((size_t)t * NG + g) * GS;
+#pragma unroll
+  for (int q = 0; q < kWideRegs; ++q) {
+    const int i = tid + 256 * q;
+    if (i < GS) o[i] = (TA)(v[q] * inv * wr[i]);
+  }
+  for (int i = tid + 256 * kWideRegs; i < GS; i += 256) {
+    const float zv = (float)zr[i];
+    o[i] = (TA)(yr[i] * zv / (1.0f + expf(-zv)) * inv * wr[i]);
+  }
+}
+
 template <typename TA>
 __global__ __launch_bounds__(256) void gate_group_norm_kernel(const float* __restrict__ y, const TA* __restrict__ z,
                                                               int ldz, const float* __restrict__ w, TA* __restrict__ out,
@@ -241,12 +343,17 @@ void gai_gated_norm_add_f32(float* res, const void* y, int ldy, int dt_y, const 
                             hipStream_t st) {
   if (T == 0) return;
   const int grid = (T + 3) / 4;
+  const bool wide = T <= 512 && D >= 512;  // few rows: a workgroup per row
 #define GAI_GNA(TY, TG, TA)                                                                                          \
-  gated_norm_add_kernel<TY, TG, TA><<<grid, 256, 0, st>>>(res, (const TY*)y, ldy, (const TG*)gate, ldg, wpost, wnext, \
-                                                          (TA*)out, T, D, eps)
-  if (dt_y && dt_gate && (dt_out || !out)) GAI_GNA(float, float, float);
-  else if (!dt_y && !dt_gate && (!dt_out || !out)) GAI_GNA(bf16, bf16, bf16);
-  else if (!dt_y && dt_gate && (!dt_out || !out)) GAI_GNA(bf16, float, bf16);
+  if (wide)                                                                                                          \
+    gated_norm_add_wide_kernel<TY, TG, TA><<<T, 256, 0, st>>>(res, (const TY*)y, ldy, (const TG*)gate, ldg, wpost,   \
+                                                              wnext, (TA*)out, D, eps);                              \
+  else                                                                                                               \
+    gated_norm_add_kernel<TY, TG, TA><<<grid, 256, 0, st>>>(res, (const TY*)y, ldy, (const TG*)gate, ldg, wpost,     \
+                                                            wnext, (TA*)out, T, D, eps)
+  if (dt_y && dt_gate && (dt_out || !out)) { GAI_GNA(float, float, float); }
+  else if (!dt_y && !dt_gate && (!dt_out || !out)) { GAI_GNA(bf16, bf16, bf16); }
+  else if (!dt_y && dt_gate && (!dt_out || !out)) { GAI_GNA(bf16, float, bf16); }
   else gai_launch_error(__FILE__, __LINE__, "gated_norm_add_f32: unsupported dtype combination");
 #undef GAI_GNA
   GAI_LAUNCH_CHECK();
@@ -256,6 +363,14 @@ void gai_gate_group_norm(const float* y, const void* z, int ldz, const float* w,
                          float eps, int dt, hipStream_t st) {
   if (T == 0) return;
   const int TG = T * NG, grid = (TG + 3) / 4;
+  if (TG <= 512 && GS >= 512) {  // few long groups: a workgroup per group
+    if (dt)
+      gate_group_norm_wide_kernel<float><<<TG, 256, 0, st>>>(y, (const float*)z, ldz, w, (float*)out, NG, GS, eps);
+    else
+      gate_group_norm_wide_kernel<bf16><<<TG, 256, 0, st>>>(y, (const bf16*)z, ldz, w, (bf16*)out, NG, GS, eps);
+    GAI_LAUNCH_CHECK();
+    return;
+  }
   if (dt)
     gate_group_norm_kernel<float><<<grid, 256, 0, st>>>(y, (const float*)z, ldz, w, (float*)out, TG, NG, GS, eps);
   else

@@ -497,16 +497,16 @@ __global__ __launch_bounds__(64) void delta_scan_cols_kernel(const float* __rest
 // thread c owns output channel c of the block for all kGT tokens and walks the block's input channels: the two weight
 // reads are coalesced over the threads ([block, in, out] layout), the u reads are LDS broadcasts. All fp32 FMA: these
 // gates steer a recurrence, so they are not rounded to the matrix cores' input format.
-constexpr int kGT = 8;
 
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
+template <int kGT>  // tokens per workgroup: 16, or fewer for wide blocks (the tile's u rows must fit in LDS)
 __global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restrict__ u, const float* __restrict__ wa_t,
                                                           const float* __restrict__ ba, const float* __restrict__ wi_t,
                                                           const float* __restrict__ bi, const float* __restrict__ lam,
                                                           float cdecay, float* __restrict__ a_out,
                                                           float* __restrict__ b_out, int T, int W, int BS) {
-  extern __shared__ float us[];  // [kGT][BS]
+  extern __shared__ __attribute__((aligned(16))) float us[];  // [kGT][BS]
   const int t0 = blockIdx.x * kGT, blk = blockIdx.y, nt = min(kGT, T - t0);
   for (int x = threadIdx.x; x < kGT * BS; x += 256) {
     const int tt = x / BS, k = x - tt * BS;
@@ -519,7 +519,30 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restric
     float ar[kGT], ai[kGT];
 #pragma unroll
     for (int tt = 0; tt < kGT; ++tt) ar[tt] = ai[tt] = 0.f;
-    for (int k = 0; k < BS; ++k) {
+    int k = 0;
+    if ((BS & 3) == 0) {  // four input channels a round: one 16-byte LDS broadcast per token instead of four reads
+      for (; k < BS; k += 4) {
+        float xa[4], xi[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          xa[q] = wa[(size_t)(k + q) * BS + c];
+          xi[q] = wi[(size_t)(k + q) * BS + c];
+        }
+#pragma unroll
+        for (int tt = 0; tt < kGT; ++tt) {
+          const float4 uv = *reinterpret_cast<const float4*>(us + tt * BS + k);
+          ar[tt] = fmaf(xa[0], uv.x, ar[tt]);
+          ai[tt] = fmaf(xi[0], uv.x, ai[tt]);
+          ar[tt] = fmaf(xa[1], uv.y, ar[tt]);
+          ai[tt] = fmaf(xi[1], uv.y, ai[tt]);
+          ar[tt] = fmaf(xa[2], uv.z, ar[tt]);
+          ai[tt] = fmaf(xi[2], uv.z, ai[tt]);
+          ar[tt] = fmaf(xa[3], uv.w, ar[tt]);
+          ai[tt] = fmaf(xi[3], uv.w, ai[tt]);
+        }
+      }
+    }
+    for (; k < BS; ++k) {
       const float xa = wa[(size_t)k * BS + c], xi = wi[(size_t)k * BS + c];
 #pragma unroll
       for (int tt = 0; tt < kGT; ++tt) {
@@ -540,6 +563,71 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restric
         a_out[o] = expf(la);
         b_out[o] = sqrtf(-expm1f(2.0f * la)) * ig * us[tt * BS + c];
       }
+    }
+  }
+}
+
+// Few tokens (decode steps): the same gates with the work of one block spread over many workgroups - one per
+// (4 tokens, block, 64 output channels), the block's input channels cut into 4 interleaved slices (one per wave) whose
+// partial sums meet in LDS - so that the gate matrices stream through all CUs instead of one workgroup per block.
+constexpr int kGS = 4;  // tokens per workgroup
+
+__global__ __launch_bounds__(256) void rglru_gates_split_kernel(const float* __restrict__ u, const float* __restrict__ wa_t,
+                                                                const float* __restrict__ ba,
+                                                                const float* __restrict__ wi_t,
+                                                                const float* __restrict__ bi, const float* __restrict__ lam,
+                                                                float cdecay, float* __restrict__ a_out,
+                                                                float* __restrict__ b_out, int T, int W, int BS) {
+  extern __shared__ __attribute__((aligned(16))) float us[];  // [kGS][BS] | red[4][2 kGS][64]
+  float* red = us + kGS * BS;
+  const int t0 = blockIdx.x * kGS, blk = blockIdx.y, c0 = blockIdx.z * 64, nt = min(kGS, T - t0);
+  const int cl = threadIdx.x & 63, ks = threadIdx.x >> 6, c = c0 + cl;
+  for (int x = threadIdx.x; x < kGS * BS; x += 256) {
+    const int tt = x / BS, k = x - tt * BS;
+    us[x] = tt < nt ? u[(size_t)(t0 + tt) * W + (size_t)blk * BS + k] : 0.f;
+  }
+  __syncthreads();
+  float ar[kGS], ai[kGS];
+#pragma unroll
+  for (int tt = 0; tt < kGS; ++tt) ar[tt] = ai[tt] = 0.f;
+  if (c < BS) {
+    const float* wa = wa_t + (size_t)blk * BS * BS + c;
+    const float* wi = wi_t + (size_t)blk * BS * BS + c;
+#pragma unroll 4
+    for (int k = ks; k < BS; k += 4) {
+      const float xa = wa[(size_t)k * BS], xi = wi[(size_t)k * BS];
+#pragma unroll
+      for (int tt = 0; tt < kGS; ++tt) {
+        const float uv = us[tt * BS + k];
+        ar[tt] = fmaf(xa, uv, ar[tt]);
+        ai[tt] = fmaf(xi, uv, ai[tt]);
+      }
+    }
+  }
+#pragma unroll
+  for (int tt = 0; tt < kGS; ++tt) {
+    red[(ks * 2 * kGS + tt) * 64 + cl] = ar[tt];
+    red[(ks * 2 * kGS + kGS + tt) * 64 + cl] = ai[tt];
+  }
+  __syncthreads();
+  if (ks != 0 || c >= BS) return;
+  const int ch = blk * BS + c;
+  const float sp = softplus_f(lam[ch]), rb = ba[ch], ib = bi[ch];
+#pragma unroll
+  for (int tt = 0; tt < kGS; ++tt) {
+    if (tt < nt) {
+      float sr = 0.f, si = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        sr += red[(q * 2 * kGS + tt) * 64 + cl];
+        si += red[(q * 2 * kGS + kGS + tt) * 64 + cl];
+      }
+      const float r = 1.0f / (1.0f + expf(-(sr + rb)));
+      const float ig = 1.0f / (1.0f + expf(-(si + ib)));
+      const float la = -cdecay * r * sp;
+      const size_t o = (size_t)(t0 + tt) * W + ch;
+      a_out[o] = expf(la);
+      b_out[o] = sqrtf(-expm1f(2.0f * la)) * ig * us[tt * BS + c];
     }
   }
 }
@@ -581,6 +669,110 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(const float* __restrict
     out[(size_t)t * ldo + c] = (TA)(scale * S * (gelu ? gelu_tanh_f(yv) : yv));
   }
   *sp = S;
+}
+
+// Prompt portions: the recurrence is linear, so a portion is cut into chunks of kChunk tokens that run side by side.
+//   pass 1 (chunk-parallel): P = product of a over the chunk, Q = the chunk's final state from a zero start;
+//   pass 2 (one thread per sequence and channel): walks the chunks, S <- P S + Q, and leaves every chunk's entry state;
+//   pass 3 (chunk-parallel): the recurrence inside the chunk from its entry state, outputs written.
+// Chunk (s, n) covers rows [cu[s] + n kChunk, ...) of sequence s; blockIdx.y walks them in sequence order.
+constexpr int kChunk = 64;
+
+__device__ __forceinline__ bool chunk_of(const int* __restrict__ cu, int S, int idx, int& s, int& t0, int& t1) {
+  int seen = 0;
+  for (s = 0; s < S; ++s) {
+    const int len = cu[s + 1] - cu[s], nc = (len + kChunk - 1) / kChunk;
+    if (idx < seen + nc) {
+      t0 = cu[s] + (idx - seen) * kChunk;
+      t1 = min(t0 + kChunk, cu[s + 1]);
+      return true;
+    }
+    seen += nc;
+  }
+  return false;
+}
+
+__global__ __launch_bounds__(256) void rglru_chunk_reduce_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                                 const int* __restrict__ cu, int S, float* __restrict__ P,
+                                                                 float* __restrict__ Q, int W) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  int s, t0, t1;
+  if (c >= W || !chunk_of(cu, S, blockIdx.y, s, t0, t1)) return;
+  float p = 1.f, q = 0.f;
+  int t = t0;
+  for (; t + 4 <= t1; t += 4) {
+    float av[4], bv[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      av[x] = a[(size_t)(t + x) * W + c];
+      bv[x] = b[(size_t)(t + x) * W + c];
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      q = fmaf(av[x], q, bv[x]);
+      p *= av[x];
+    }
+  }
+  for (; t < t1; ++t) {
+    const float av = a[(size_t)t * W + c];
+    q = fmaf(av, q, b[(size_t)t * W + c]);
+    p *= av;
+  }
+  P[(size_t)blockIdx.y * W + c] = p;
+  Q[(size_t)blockIdx.y * W + c] = q;
+}
+
+__global__ __launch_bounds__(256) void rglru_chunk_carry_kernel(const float* __restrict__ P, const float* __restrict__ Q,
+                                                                float* __restrict__ Sin, float* __restrict__ state,
+                                                                const int* __restrict__ cu, const int* __restrict__ slots,
+                                                                int W) {
+  const int s = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  if (c >= W) return;
+  const int len = cu[s + 1] - cu[s];
+  if (len <= 0) return;
+  int first = 0;
+  for (int x = 0; x < s; ++x) first += (cu[x + 1] - cu[x] + kChunk - 1) / kChunk;
+  const int nc = (len + kChunk - 1) / kChunk;
+  float* sp = state + (size_t)slots[s] * W + c;
+  float Sv = *sp;
+  for (int n = 0; n < nc; ++n) {
+    const size_t o = (size_t)(first + n) * W + c;
+    Sin[o] = Sv;
+    Sv = fmaf(P[o], Sv, Q[o]);
+  }
+  *sp = Sv;
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void rglru_chunk_apply_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                                const TA* __restrict__ y, int ldy,
+                                                                const float* __restrict__ Sin, const int* __restrict__ cu,
+                                                                int S, TA* __restrict__ out, int ldo, int W, int gelu,
+                                                                float scale) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  int s, t0, t1;
+  if (c >= W || !chunk_of(cu, S, blockIdx.y, s, t0, t1)) return;
+  float Sv = Sin[(size_t)blockIdx.y * W + c];
+  int t = t0;
+  for (; t + 4 <= t1; t += 4) {
+    float av[4], bv[4], yv[4];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      av[x] = a[(size_t)(t + x) * W + c];
+      bv[x] = b[(size_t)(t + x) * W + c];
+      yv[x] = (float)y[(size_t)(t + x) * ldy + c];
+    }
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      Sv = fmaf(av[x], Sv, bv[x]);
+      out[(size_t)(t + x) * ldo + c] = (TA)(scale * Sv * (gelu ? gelu_tanh_f(yv[x]) : yv[x]));
+    }
+  }
+  for (; t < t1; ++t) {
+    Sv = fmaf(a[(size_t)t * W + c], Sv, b[(size_t)t * W + c]);
+    const float yv = (float)y[(size_t)t * ldy + c];
+    out[(size_t)t * ldo + c] = (TA)(scale * Sv * (gelu ? gelu_tanh_f(yv) : yv));
+  }
 }
 
 // ---- state-space scan with a scalar decay per head ----------------------------------------------------------------
@@ -859,16 +1051,45 @@ void gai_rglru_gates(const float* u, const float* wa_t, const float* ba, const f
   if (T == 0) return;
   if (NB < 1 || W % NB) gai_launch_error(__FILE__, __LINE__, "rglru_gates: width must be a multiple of the blocks");
   const int BS = W / NB;
-  const size_t lds = (size_t)kGT * BS * sizeof(float);
-  if (lds > 64 * 1024) gai_launch_error(__FILE__, __LINE__, "rglru_gates: block size above 2048");
-  const dim3 grid((T + kGT - 1) / kGT, NB);
-  rglru_gates_kernel<<<grid, 256, lds, st>>>(u, wa_t, ba, wi_t, bi, lam, cdecay, a_out, b_out, T, W, BS);
+  if (BS > 3584) gai_launch_error(__FILE__, __LINE__, "rglru_gates: block size above 3584");
+  if (T <= 64 && BS <= 3072) {  // decode-sized steps
+    const dim3 grid((T + kGS - 1) / kGS, NB, (BS + 63) / 64);
+    const size_t lds2 = (size_t)(kGS * BS + 4 * 2 * kGS * 64) * sizeof(float);
+    rglru_gates_split_kernel<<<grid, 256, lds2, st>>>(u, wa_t, ba, wi_t, bi, lam, cdecay, a_out, b_out, T, W, BS);
+    GAI_LAUNCH_CHECK();
+    return;
+  }
+#define GAI_GATES(GT)                                                                                                \
+  rglru_gates_kernel<GT><<<dim3((T + GT - 1) / GT, NB), 256, (size_t)GT * BS * sizeof(float), st>>>(                 \
+      u, wa_t, ba, wi_t, bi, lam, cdecay, a_out, b_out, T, W, BS)
+  if (BS <= 1024) GAI_GATES(16); else if (BS <= 2048) GAI_GATES(8); else GAI_GATES(4);
+#undef GAI_GATES
   GAI_LAUNCH_CHECK();
 }
 
+int gai_rglru_scan_chunks(int T, int S) { return T / kChunk + S; }
+
 void gai_rglru_scan(const float* a, const float* b, const void* y, int ldy, float* state, const int* cu,
-                    const int* slots, int S, void* out, int ldo, int W, int gelu, float scale, int dt, hipStream_t st) {
-  if (S == 0) return;
+                    const int* slots, int S, int T, void* out, int ldo, int W, int gelu, float scale, int dt, float* ws,
+                    hipStream_t st) {
+  if (S == 0 || T == 0) return;
+  if (T > S && ws) {  // some sequence brings more than one row: chunk-parallel scan (ws: [3][T / kChunk + S][W])
+    const int NC = gai_rglru_scan_chunks(T, S);
+    float* P = ws;
+    float* Q = ws + (size_t)NC * W;
+    float* Sin = ws + 2 * (size_t)NC * W;
+    const dim3 gc((W + 255) / 256, NC), gs((W + 255) / 256, S);
+    rglru_chunk_reduce_kernel<<<gc, 256, 0, st>>>(a, b, cu, S, P, Q, W);
+    rglru_chunk_carry_kernel<<<gs, 256, 0, st>>>(P, Q, Sin, state, cu, slots, W);
+    if (dt)
+      rglru_chunk_apply_kernel<float><<<gc, 256, 0, st>>>(a, b, (const float*)y, ldy, Sin, cu, S, (float*)out, ldo, W,
+                                                          gelu, scale);
+    else
+      rglru_chunk_apply_kernel<bf16><<<gc, 256, 0, st>>>(a, b, (const bf16*)y, ldy, Sin, cu, S, (bf16*)out, ldo, W, gelu,
+                                                         scale);
+    GAI_LAUNCH_CHECK();
+    return;
+  }
   const dim3 grid((W + 255) / 256, S);
   if (dt)
     rglru_scan_kernel<float><<<grid, 256, 0, st>>>(a, b, (const float*)y, ldy, state, cu, slots, (float*)out, ldo, W,

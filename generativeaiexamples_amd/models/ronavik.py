@@ -25,7 +25,7 @@ cache layer per ``parallel`` layer, each with its own head geometry); the recurr
 (convolution tails, S vectors / matrices) in the engine's state slot pool. A step's rows - prompt portions and single
 decoded tokens alike - go through the same HIP kernels, addressed by device-side (cu, slot, ctx) vectors, so
 pure-decode steps replay a captured HIP graph. Per layer the projections that read the same input are one GEMM
-(q | k | v | y | x | residual gate; in | residual gate; residual gate | router), the two output projections of a
+(q | k | v | y | x | residual gate; in | residual gate), the two output projections of a
 ``parallel`` mixer are one GEMM over the concatenated branch outputs, and the closing norm of a sublayer is fused with
 the residual add and the opening norm of the next sublayer.
 """
@@ -280,8 +280,10 @@ class RonavikModel:
                 E = ml["router"]["experts"]
                 for k in ("norm2", "norm2b"):
                     w[p + k] = f32(sd[p + k])
-                w[p + "rg2r"] = mat(torch.cat([sd[p + "rg2"], sd[p + "mlp.router"]]))
-                w[p + "rg2r.b"] = mat(torch.cat([sd[p + "rg2.b"].float(), torch.zeros(E)]))
+                w[p + "rg2"], w[p + "rg2.b"] = mat(sd[p + "rg2"]), mat(sd[p + "rg2.b"])
+                # router rows padded to the GEMM's 16-column grid: the logits come out of the MFMA kernel in fp32
+                pad = (-E) % 16
+                w[p + "mlp.router"] = mat(torch.cat([sd[p + "mlp.router"].float(), torch.zeros(pad, D)]))
                 w[p + "mlp.up"] = mat(torch.stack([sd[p + f"mlp.e{e}.up"] for e in range(E)]))
                 w[p + "mlp.down"] = mat(torch.stack([sd[p + f"mlp.e{e}.down"] for e in range(E)]))
         self._alloc_state()
@@ -414,14 +416,15 @@ class RonavikModel:
         """-> (feed-forward output, residual-gate logits)."""
         ml, w, p = self.cfg.layers[i]["mlp"], self.w, f"l{i}."
         D, E, top = self.cfg.hidden_size, ml["router"]["experts"], ml["router"]["top"]
-        gr = ops.linear(h, w[p + "rg2r"], w[p + "rg2r.b"], out_dtype=torch.float32)
-        ids, wts = ops.moe_route(gr[:, D:], top, renorm=False, score="sigmoid")
+        gate = ops.linear(h, w[p + "rg2"], w[p + "rg2.b"])
+        logits = ops.linear(h, w[p + "mlp.router"], out_dtype=torch.float32)[:, :E]
+        ids, wts = ops.moe_route(logits, top, renorm=False, score="sigmoid")
         _rows, offs, pos = ops.moe_dispatch(ids, E)
         xs = ops.moe_scale_rows(h, pos, wts)
         n = h.shape[0] * top
         up = ops.moe_gemm(xs, None, w[p + "mlp.up"], offs, n, act="relu2")
         dn = ops.moe_gemm(up, None, w[p + "mlp.down"], offs, n)
-        return ops.moe_combine(dn, pos, None), gr[:, :D]
+        return ops.moe_combine(dn, pos, None), gate
 
     # ------------------------------------------------------------------ forward
     def forward(self, fb: ForwardBatch, kv, decode_ws=None) -> torch.Tensor:

@@ -1231,7 +1231,10 @@ def rglru_scan(a, b, y, state, cu, slots, out_dtype, act: Optional[str] = None, 
         return _into(out, ref.rglru_scan(a, b, y, state, cu, slots, out_dtype, act, out_scale))
     if out is None:
         out = torch.empty(a.shape, dtype=out_dtype, device=a.device)
-    native().rglru_scan(a, b, y, state, cu, slots, out, act == "gelu_tanh", float(out_scale))
+    # a step with prompt portions (more rows than sequences) runs the chunk-parallel scan through a scratch
+    T, S, W = a.shape[0], slots.numel(), a.shape[1]
+    ws = torch.empty(native().rglru_scan_ws_floats(T, S, W), dtype=torch.float32, device=a.device) if T > S else None
+    native().rglru_scan(a, b, y, state, cu, slots, out, act == "gelu_tanh", float(out_scale), ws)
     return out
 
 

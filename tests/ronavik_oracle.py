@@ -112,11 +112,14 @@ def mamba2_mixer(h, W, p, m, eps):
     return y @ W[p + "o"].T
 
 
-def moe(h, W, p, ml):
+def moe(h, W, p, ml, gaps=None):
     """Sigmoid router; the chosen experts' scores scale each expert's INPUT; experts are W_down relu(W_up .)^2."""
     T = h.shape[0]
     E, top = ml["router"]["experts"], ml["router"]["top"]
     s = torch.sigmoid(h @ W[p + "router"].T)
+    if gaps is not None and top < E:
+        ss = s.sort(-1, descending=True).values
+        gaps.append(float((ss[:, top - 1] - ss[:, top]).min()))
     out = torch.zeros(T, W[p + "e0.down"].shape[0], dtype=F64)
     for t in range(T):
         order = sorted(range(E), key=lambda e: (-float(s[t, e]), e))[:top]
@@ -126,7 +129,7 @@ def moe(h, W, p, ml):
     return out
 
 
-def forward(cfg: dict, W: dict, tokens, residuals: list | None = None):
+def forward(cfg: dict, W: dict, tokens, residuals: list | None = None, gaps: list | None = None):
     """tokens: list of ints -> logits [T, vocab] (float64). `residuals` collects the stream after every layer."""
     W = {k: v.to(F64) if v.is_floating_point() else v for k, v in W.items()}
     eps = cfg["norm"]["eps"]
@@ -145,9 +148,100 @@ def forward(cfg: dict, W: dict, tokens, residuals: list | None = None):
         x = x + norm(y, W[p + "norm1b"], eps)
         if l.get("mlp") is not None:
             h = norm(x, W[p + "norm2"], eps)
-            y = moe(h, W, p + "mlp.", l["mlp"])
+            y = moe(h, W, p + "mlp.", l["mlp"], gaps)
             y = y * torch.sigmoid(h @ W[p + "rg2"].T + W[p + "rg2.b"])
             x = x + norm(y, W[p + "norm2b"], eps)
         if residuals is not None:
             residuals.append(x.clone())
     return norm(x, W["final.norm"], eps) @ W["embed"].T
+
+
+# ------------------------------------------------------------------------------------------------ test model builders
+def par(dim=8, vdim=12, heads=4, kv_heads=2, scale=0.35, q_temp=(0.5, 4), width=24, blocks=3, conv=3, left_scale=0.7,
+        right_scale=1.4):
+    left = dict(dim=dim, vdim=vdim, heads=heads, kv_heads=kv_heads, scale=scale)
+    if q_temp:
+        left["q_temp"] = dict(coef=q_temp[0], every=q_temp[1])
+    return dict(type="parallel", mixer=dict(left=left, right=dict(width=width, blocks=blocks, conv=conv),
+                                            left_scale=left_scale, right_scale=right_scale))
+
+
+def ssm(heads=4, vdim=8, state=12, groups=2, norm_groups=4, conv=4):
+    return dict(type="mamba2", mixer=dict(heads=heads, vdim=vdim, state=state, groups=groups, norm_groups=norm_groups,
+                                          conv=conv))
+
+
+def with_mlp(layer, ff=24, experts=5, top=2):
+    mlp = None if ff is None else dict(kind="moe", expert=dict(ff=ff), router=dict(experts=experts, top=top))
+    return dict(layer, mlp=mlp)
+
+
+def make_config(layers, width=32, vocab=97, eps=1e-5, max_positions=400):
+    return dict(architecture="Ronavik", vocab=vocab, width=width, max_positions=max_positions, norm=dict(eps=eps),
+                layers=list(layers))
+
+
+def random_checkpoint(cfg, seed, slow_decay=False):
+    """Random weights under the checkpoint's tensor names, rounded to bfloat16 (what a stored checkpoint holds), with
+    magnitudes that make every mechanism matter: sizeable position vectors, biases, gate matrices and routers."""
+    g = torch.Generator().manual_seed(seed)
+    D = cfg["width"]
+
+    def rn(*s, std=1.0):
+        return (torch.randn(*s, generator=g) * std).to(torch.bfloat16).float()
+
+    def un(*s, lo=0.0, hi=1.0):
+        return (torch.rand(*s, generator=g) * (hi - lo) + lo).to(torch.bfloat16).float()
+
+    def lin(o, i, gain=1.0):
+        return rn(o, i, std=gain * i ** -0.5)
+
+    W = {"embed": rn(cfg["vocab"], D), "pos": rn(cfg["max_positions"], D, std=0.5), "final.norm": un(D, lo=0.5, hi=1.5)}
+    for i, l in enumerate(cfg["layers"]):
+        p, x, m = f"l{i}.", f"l{i}.mix.", l["mixer"]
+        W[p + "norm1"], W[p + "norm1b"] = un(D, lo=0.5, hi=1.5), un(D, lo=0.5, hi=1.5)
+        W[p + "rg1"], W[p + "rg1.b"] = lin(D, D, 2.0), rn(D)
+        if l["type"] == "parallel":
+            a, r = m["left"], m["right"]
+            H, G, dk, dv = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            xl, xr = x + "left.", x + "right."
+            W[xl + "q"], W[xl + "k"], W[xl + "v"] = lin(H * dk, D, 2.0), lin(G * dk, D, 2.0), lin(G * dv, D)
+            W[xl + "q.norm"], W[xl + "k.norm"] = un(dk, lo=0.5, hi=1.5), un(dk, lo=0.5, hi=1.5)
+            W[xl + "pb"] = un(H, lo=-3.0, hi=0.0)
+            W[xl + "o"] = lin(D, H * dv)
+            Wd, nb, K = r["width"], r["blocks"], r["conv"]
+            bs = Wd // nb
+            W[xr + "y"], W[xr + "y.b"] = lin(Wd, D), rn(Wd, std=0.3)
+            W[xr + "x"], W[xr + "x.b"] = lin(Wd, D), rn(Wd, std=0.3)
+            W[xr + "conv"], W[xr + "conv.b"] = rn(Wd, K, std=0.6), rn(Wd, std=0.2)
+            W[xr + "ra"], W[xr + "ra.b"] = rn(nb, bs, bs, std=2.0 * bs ** -0.5), rn(nb, bs)
+            W[xr + "ri"], W[xr + "ri.b"] = rn(nb, bs, bs, std=2.0 * bs ** -0.5), rn(nb, bs)
+            W[xr + "lam"] = un(Wd, lo=-9.0, hi=-6.0) if slow_decay else un(Wd, lo=-4.0, hi=0.5)
+            W[xr + "o"] = lin(D, Wd)
+        else:
+            H, dv, N, G, K = m["heads"], m["vdim"], m["state"], m["groups"], m["conv"]
+            inner, C = H * dv, H * dv + 2 * G * N
+            W[x + "in"] = lin(2 * inner + 2 * G * N + H, D, 1.5)
+            W[x + "conv"], W[x + "conv.b"] = rn(C, K, std=0.6), rn(C, std=0.2)
+            W[x + "dt_bias"] = un(H, lo=-6.0, hi=-4.0) if slow_decay else un(H, lo=-2.0, hi=1.0)
+            W[x + "A_log"] = un(H, lo=-2.0, hi=-1.0) if slow_decay else un(H, lo=-1.0, hi=1.2)
+            W[x + "D"] = rn(H)
+            W[x + "norm"] = un(inner, lo=0.5, hi=1.5)
+            W[x + "o"] = lin(D, inner)
+        ml = l.get("mlp")
+        if ml is not None:
+            F_, E = ml["expert"]["ff"], ml["router"]["experts"]
+            W[p + "norm2"], W[p + "norm2b"] = un(D, lo=0.5, hi=1.5), un(D, lo=0.5, hi=1.5)
+            W[p + "rg2"], W[p + "rg2.b"] = lin(D, D, 2.0), rn(D)
+            W[p + "mlp.router"] = lin(E, D, 3.0)
+            for e in range(E):
+                W[p + f"mlp.e{e}.up"], W[p + f"mlp.e{e}.down"] = lin(F_, D, 1.5), lin(D, F_)
+    return W
+
+
+def router_margin(cfg, W, tokens):
+    """Smallest gap between the last chosen and the first not chosen router score over all layers and positions (a test
+    with a near-tie would rest on rounding)."""
+    gaps = []
+    forward(cfg, W, tokens, gaps=gaps)
+    return min(gaps) if gaps else 1.0
