@@ -273,9 +273,13 @@ void rglru_scan(const Tensor& a, const Tensor& b, const Tensor& y, Tensor& state
                  dt, wsp, cur_stream());
 }
 
+int64_t ssd_scan_ws_floats(int64_t T, int64_t S, int64_t H, int64_t N, int64_t DV) {
+  return (int64_t)gai_ssd_scan_ws_floats(T, S, H, N, DV);
+}
+
 void ssd_scan(const Tensor& x, const Tensor& B, const Tensor& C, const Tensor& dt, const Tensor& dt_bias,
               const Tensor& A_log, const Tensor& D, Tensor& state, const Tensor& cu, const Tensor& slots, Tensor& out,
-              int64_t G) {
+              int64_t G, const optional<Tensor>& ws) {
   TORCH_CHECK(state.dim() == 4, "ssd_scan: state [slots, H, N, DV]");
   const int H = state.size(1), N = state.size(2), DV = state.size(3), S = slots.numel();
   auto f32row = [](const Tensor& t, const char* name) {
@@ -290,9 +294,15 @@ void ssd_scan(const Tensor& x, const Tensor& B, const Tensor& C, const Tensor& d
                   dt.size(0) == T && dt.size(1) == H && dt_bias.numel() == H && A_log.numel() == H && D.numel() == H &&
                   cu.numel() == S + 1 && out.numel() == (int64_t)T * H * DV && G >= 1 && H % G == 0,
               "ssd_scan: shapes");
+  float* wsp = nullptr;
+  if (ws) {
+    TORCH_CHECK(ws->is_cuda() && ws->scalar_type() == at::kFloat && ws->is_contiguous() &&
+                    ws->numel() >= ssd_scan_ws_floats(T, S, H, N, DV), "ssd_scan: workspace too small");
+    wsp = ws->data_ptr<float>();
+  }
   gai_ssd_scan(x.data_ptr<float>(), B.data_ptr<float>(), C.data_ptr<float>(), ld, dt.data_ptr(), row_stride(dt, "dt"),
                f32(dt_bias, "dt_bias"), f32(A_log, "A_log"), f32(D, "D"), f32w(state, "state"), i32(cu, "cu"),
-               i32(slots, "slots"), S, T, f32w(out, "out"), H, (int)G, N, DV, dtt, cur_stream());
+               i32(slots, "slots"), S, T, f32w(out, "out"), H, (int)G, N, DV, dtt, wsp, cur_stream());
 }
 
 void wkv_scan(const Tensor& r, const Tensor& k, const Tensor& v, const Tensor& wpre, const Tensor& w0, const Tensor& u,
@@ -372,4 +382,5 @@ void gai_bind_seq_ops(pybind11::module_& m) {
   m.def("rglru_scan", &rglru_scan);
   m.def("rglru_scan_ws_floats", &rglru_scan_ws_floats);
   m.def("ssd_scan", &ssd_scan);
+  m.def("ssd_scan_ws_floats", &ssd_scan_ws_floats);
 }

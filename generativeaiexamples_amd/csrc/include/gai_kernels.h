@@ -249,7 +249,10 @@ void gai_rglru_scan(const float* a, const float* b, const void* y, int ldy, floa
                     hipStream_t st);
 void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const void* dt, int lddt,
                   const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu,
-                  const int* slots, int S, int T, float* out, int H, int G, int N, int DV, int dtt, hipStream_t st);
+                  const int* slots, int S, int T, float* out, int H, int G, int N, int DV, int dtt, float* ws,
+                  hipStream_t st);
+// scratch (fp32 elements) for the chunk-parallel form of a step with long portions of few sequences; 0: not chunked
+size_t gai_ssd_scan_ws_floats(int T, int S, int H, int N, int DV);
 void gai_wkv_scan(const void* r, const void* k, const void* v, int ld, const float* wpre, const float* w0,
                   const float* u, float* state, const int* cu, const int* slots, int S, int T, float* out, int H, int D,
                   int dt, float* ws, hipStream_t st);

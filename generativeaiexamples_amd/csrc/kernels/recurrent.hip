@@ -678,13 +678,14 @@ __global__ __launch_bounds__(256) void rglru_scan_kernel(const float* __restrict
 // Chunk (s, n) covers rows [cu[s] + n kChunk, ...) of sequence s; blockIdx.y walks them in sequence order.
 constexpr int kChunk = 64;
 
+template <int L = kChunk>
 __device__ __forceinline__ bool chunk_of(const int* __restrict__ cu, int S, int idx, int& s, int& t0, int& t1) {
   int seen = 0;
   for (s = 0; s < S; ++s) {
-    const int len = cu[s + 1] - cu[s], nc = (len + kChunk - 1) / kChunk;
+    const int len = cu[s + 1] - cu[s], nc = (len + L - 1) / L;
     if (idx < seen + nc) {
-      t0 = cu[s] + (idx - seen) * kChunk;
-      t1 = min(t0 + kChunk, cu[s + 1]);
+      t0 = cu[s] + (idx - seen) * L;
+      t1 = min(t0 + L, cu[s + 1]);
       return true;
     }
     seen += nc;
@@ -837,7 +838,15 @@ __global__ __launch_bounds__(1024) void ssd_scan_kernel(const float* __restrict_
     if (i < nrow) Sg[(size_t)i * DV] = col[i];
 }
 
-template <typename TA, int R, int RGS>
+// MODE 0: whole portions, state from / to the pool. A long portion of few sequences leaves most SIMDs with one wave
+// and nothing to hide its latencies behind; the recurrence is linear in S (one scalar decay per head and token), so such
+// a step is cut into chunks of kSsdChunk tokens that run side by side:
+//   MODE 1: a chunk from a zero state, no outputs: its final state Q and the product P of its decays;
+//   carry:  per sequence S <- P S + Q over its chunks, leaving every chunk's entry state (and the pool's final state);
+//   MODE 2: the chunk again from its entry state, outputs written.
+constexpr int kSsdChunk = 256;
+
+template <typename TA, int R, int RGS, int MODE>
 __global__ __launch_bounds__(64) void ssd_scan_cols_kernel(const float* __restrict__ x, const float* __restrict__ Bm,
                                                            const float* __restrict__ Cm, int ld,
                                                            const TA* __restrict__ dt, int lddt,
@@ -845,10 +854,18 @@ __global__ __launch_bounds__(64) void ssd_scan_cols_kernel(const float* __restri
                                                            const float* __restrict__ A_log,
                                                            const float* __restrict__ Dskip, float* __restrict__ state,
                                                            const int* __restrict__ cu, const int* __restrict__ slots,
-                                                           float* __restrict__ out, int H, int G, int N, int DV) {
+                                                           float* __restrict__ out, int H, int G, int N, int DV, int S,
+                                                           float* __restrict__ Pbuf, float* __restrict__ Qbuf) {
   constexpr int COLS = 64 / RGS, NP = kTB * RGS * R / 64, LD = RGS * R + RGS;
   extern __shared__ float lds[];
-  const int h = blockIdx.x, s = blockIdx.y, cb = blockIdx.z, lane = threadIdx.x;
+  const int h = blockIdx.x, cb = blockIdx.z, lane = threadIdx.x;
+  int s = blockIdx.y, t0, t1;
+  if (MODE == 0) {
+    t0 = cu[s];
+    t1 = cu[s + 1];
+  } else if (!chunk_of<kSsdChunk>(cu, S, blockIdx.y, s, t0, t1)) {
+    return;
+  }
   const int jj = lane / RGS, rg = lane % RGS, j = cb * COLS + jj;
   const bool on = j < DV;
   const int row0 = rg * R, nrow = max(0, min(R, N - row0));
@@ -857,13 +874,15 @@ __global__ __launch_bounds__(64) void ssd_scan_cols_kernel(const float* __restri
   float* Cs = Bs + kTB * LD;
   float* xs = Cs + kTB * LD;     // [kTB][COLS]
   float* ds = xs + kTB * COLS;   // [2][kTB]: step size, decay
-  const int t0 = cu[s], t1 = cu[s + 1];
   if (t1 <= t0) return;
   for (int q = lane; q < 2 * kTB * LD; q += 64) lds[q] = 0.f;
-  float* Sg = state + (((size_t)slots[s] * H + h) * N + row0) * DV + j;
+  // MODE 0: the pool's slot; MODE 1 / 2: the chunk's own [H, N, DV] image in Qbuf (MODE 2 reads its entry state there)
+  float* Sg = (MODE == 0 ? state + (((size_t)slots[s] * H + h) * N + row0) * DV
+                         : Qbuf + (((size_t)blockIdx.y * H + h) * N + row0) * DV) + j;
   float col[R];
+  float pprod = 1.f;
 #pragma unroll
-  for (int i = 0; i < R; ++i) col[i] = (on && i < nrow) ? Sg[(size_t)i * DV] : 0.f;
+  for (int i = 0; i < R; ++i) col[i] = (MODE != 1 && on && i < nrow) ? Sg[(size_t)i * DV] : 0.f;
   const float negA = -expf(A_log[h]), dskip = Dskip[h], dtb = dt_bias[h];
   constexpr int NPART = 64 / kTB;
   static_assert(NP * NPART >= RGS * R, "staging covers a full row");
@@ -923,15 +942,42 @@ __global__ __launch_bounds__(64) void ssd_scan_cols_kernel(const float* __restri
         acc0 = fmaf(col[i], Cs[a + i], acc0);
         acc1 = fmaf(col[i + 1], Cs[a + i + 1], acc1);
       }
-      const float acc = rowgroup_sum<RGS>(acc0 + acc1);
-      if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * DV + j] = fmaf(dskip, xj, acc);
+      if (MODE == 1) {
+        pprod *= dec;
+      } else {
+        const float acc = rowgroup_sum<RGS>(acc0 + acc1);
+        if (rg == 0 && on) out[((size_t)(tb + tt) * H + h) * DV + j] = fmaf(dskip, xj, acc);
+      }
     }
   }
-  if (on) {
+  if (MODE != 2 && on) {
 #pragma unroll
     for (int i = 0; i < R; ++i)
       if (i < nrow) Sg[(size_t)i * DV] = col[i];
   }
+  if (MODE == 1 && cb == 0 && lane == 0) Pbuf[(size_t)blockIdx.y * H + h] = pprod;
+}
+
+// S <- P S + Q over the chunks of a sequence; Q[chunk] is replaced by the chunk's entry state
+__global__ __launch_bounds__(256) void ssd_chunk_carry_kernel(const float* __restrict__ Pbuf, float* __restrict__ Qbuf,
+                                                              float* __restrict__ state, const int* __restrict__ cu,
+                                                              const int* __restrict__ slots, int H, int ND) {
+  const int e = blockIdx.x * 256 + threadIdx.x, h = blockIdx.y, s = blockIdx.z;
+  if (e >= ND) return;
+  const int len = cu[s + 1] - cu[s];
+  if (len <= 0) return;
+  int first = 0;
+  for (int q = 0; q < s; ++q) first += (cu[q + 1] - cu[q] + kSsdChunk - 1) / kSsdChunk;
+  const int nc = (len + kSsdChunk - 1) / kSsdChunk;
+  float* sp = state + ((size_t)slots[s] * H + h) * ND + e;
+  float Sv = *sp;
+  for (int n = 0; n < nc; ++n) {
+    float* qp = Qbuf + ((size_t)(first + n) * H + h) * ND + e;
+    const float q = *qp;
+    *qp = Sv;
+    Sv = fmaf(Pbuf[(size_t)(first + n) * H + h], Sv, q);
+  }
+  *sp = Sv;
 }
 
 }  // namespace
@@ -1100,19 +1146,45 @@ void gai_rglru_scan(const float* a, const float* b, const void* y, int ldy, floa
   GAI_LAUNCH_CHECK();
 }
 
+// fp32 elements of the scratch that the chunked scan of such a step needs (0: the step runs unchunked)
+size_t gai_ssd_scan_ws_floats(int T, int S, int H, int N, int DV) {
+  const int RGS = N <= 64 ? 8 : 16;
+  const long waves = (long)H * S * ((DV + 64 / RGS - 1) / (64 / RGS));
+  if (T <= S || T < 2 * kSsdChunk || waves >= 4096) return 0;  // single tokens, short portions, or SIMDs already full
+  const size_t NC = (size_t)T / kSsdChunk + S;
+  return NC * H * ((size_t)N * DV + 1);
+}
+
 void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const void* dt, int lddt,
                   const float* dt_bias, const float* A_log, const float* D, float* state, const int* cu,
-                  const int* slots, int S, int T, float* out, int H, int G, int N, int DV, int dtt, hipStream_t st) {
+                  const int* slots, int S, int T, float* out, int H, int G, int N, int DV, int dtt, float* ws,
+                  hipStream_t st) {
   if (S == 0) return;
   if (H % G) gai_launch_error(__FILE__, __LINE__, "ssd_scan: heads must be a multiple of groups");
   if (N > kMaxDK) gai_launch_error(__FILE__, __LINE__, "ssd_scan: state size above 256");
   if (T > S) {  // some sequence brings more than one row: the column-sliced scan
+    const bool chunked = ws && gai_ssd_scan_ws_floats(T, S, H, N, DV) > 0;
+    const int NC = T / kSsdChunk + S;
+    float* Qbuf = ws;
+    float* Pbuf = ws ? ws + (size_t)NC * H * N * DV : nullptr;
+#define GAI_SSD_L(TA, R, RGS, MODE, NY)                                                                              \
+  do {                                                                                                               \
+    const dim3 grid(H, NY, (DV + 64 / RGS - 1) / (64 / RGS));                                                        \
+    const size_t lds = (size_t)(2 * kTB * (RGS * R + RGS) + kTB * (64 / RGS) + 2 * kTB) * sizeof(float);             \
+    ssd_scan_cols_kernel<TA, R, RGS, MODE><<<grid, 64, lds, st>>>(x, B, C, ld, (const TA*)dt, lddt, dt_bias, A_log,  \
+                                                                  D, state, cu, slots, out, H, G, N, DV, S, Pbuf,   \
+                                                                  Qbuf);                                             \
+  } while (0)
 #define GAI_SSD(TA, R, RGS)                                                                                          \
   do {                                                                                                               \
-    const dim3 grid(H, S, (DV + 64 / RGS - 1) / (64 / RGS));                                                         \
-    const size_t lds = (size_t)(2 * kTB * (RGS * R + RGS) + kTB * (64 / RGS) + 2 * kTB) * sizeof(float);             \
-    ssd_scan_cols_kernel<TA, R, RGS><<<grid, 64, lds, st>>>(x, B, C, ld, (const TA*)dt, lddt, dt_bias, A_log, D,    \
-                                                            state, cu, slots, out, H, G, N, DV);                    \
+    if (chunked) {                                                                                                   \
+      GAI_SSD_L(TA, R, RGS, 1, NC);                                                                                  \
+      ssd_chunk_carry_kernel<<<dim3((N * DV + 255) / 256, H, S), 256, 0, st>>>(Pbuf, Qbuf, state, cu, slots, H,      \
+                                                                                N * DV);                             \
+      GAI_SSD_L(TA, R, RGS, 2, NC);                                                                                  \
+    } else {                                                                                                         \
+      GAI_SSD_L(TA, R, RGS, 0, S);                                                                                   \
+    }                                                                                                                \
   } while (0)
     if (dtt) {
       if (N <= 64) GAI_SSD(float, 8, 8); else if (N <= 128) GAI_SSD(float, 8, 16); else GAI_SSD(float, 16, 16);
@@ -1120,6 +1192,7 @@ void gai_ssd_scan(const float* x, const float* B, const float* C, int ld, const 
       if (N <= 64) GAI_SSD(bf16, 8, 8); else if (N <= 128) GAI_SSD(bf16, 8, 16); else GAI_SSD(bf16, 16, 16);
     }
 #undef GAI_SSD
+#undef GAI_SSD_L
     GAI_LAUNCH_CHECK();
     return;
   }

@@ -1247,7 +1247,10 @@ def ssd_scan(x, B, C, dt, dt_bias, A_log, D, state, cu, slots, G: int):
         return ref.ssd_scan(x, B, C, dt, dt_bias, A_log, D, state, cu, slots, G)
     H, DV = state.shape[1], state.shape[3]
     out = torch.empty(x.shape[0], H, DV, dtype=torch.float32, device=x.device)
-    native().ssd_scan(x, B, C, dt, dt_bias, A_log, D, state, cu, slots, out, G)
+    # long portions of few sequences run chunk-parallel through a scratch (chunk states and decay products)
+    nws = native().ssd_scan_ws_floats(x.shape[0], slots.numel(), H, state.shape[2], DV)
+    ws = torch.empty(nws, dtype=torch.float32, device=x.device) if nws else None
+    native().ssd_scan(x, B, C, dt, dt_bias, A_log, D, state, cu, slots, out, G, ws)
     return out
 
 

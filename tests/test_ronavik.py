@@ -510,3 +510,17 @@ def test_kernel_shape_variants(dtype):
     o1 = ops.rglru_scan(a, b, yv[:, 8:], s1, cu, slots, dtype, act="gelu_tanh", out_scale=1.1)
     o2 = ops.rglru_scan(a.cuda(), b.cuda(), yv.cuda()[:, 8:], s2, cu.cuda(), slots.cuda(), dtype, act="gelu_tanh", out_scale=1.1)
     assert rel(o2, o1) < lim and rel(s2, s1) < 1e-5
+    # state-space scan: long portions of few sequences take the chunk-parallel form (several chunks, a single token
+    # between them, a state that does not start at zero)
+    for (H, G, N, DV) in ((4, 2, 32, 32), (2, 1, 100, 24)):
+        inner, T = H * DV, 1300
+        cu = torch.tensor([0, 600, 601, 1300], dtype=torch.int32)
+        slots = torch.tensor([1, 3, 0], dtype=torch.int32)
+        cv, dtr = rn(T, inner + 2 * G * N) * 0.5, rn(T, H + 3).to(dtype)
+        dtb, A, Dk, st = rn(H) - 1, rn(H) * 0.5, rn(H), rn(4, H, N, DV) * 0.3
+        s1, s2, cg, dg = st.clone(), st.clone().cuda(), cv.cuda(), dtr.cuda()
+        o1 = ops.ssd_scan(cv[:, :inner], cv[:, inner:inner + G * N], cv[:, inner + G * N:], dtr[:, 1:H + 1], dtb, A, Dk, s1,
+                          cu, slots, G)
+        o2 = ops.ssd_scan(cg[:, :inner], cg[:, inner:inner + G * N], cg[:, inner + G * N:], dg[:, 1:H + 1], dtb.cuda(),
+                          A.cuda(), Dk.cuda(), s2, cu.cuda(), slots.cuda(), G)
+        assert rel(o2, o1) < 5e-5 and rel(s2, s1) < 5e-5, (H, G, N, DV)
