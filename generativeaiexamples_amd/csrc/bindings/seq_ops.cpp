@@ -179,7 +179,7 @@ void window_attention(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
                       const Tensor& cu_q, const Tensor& ctx, Tensor& out, int64_t H, int64_t G, int64_t DK, int64_t DV,
                       double scale, double softcap, int64_t window, const optional<Tensor>& r1,
                       const optional<Tensor>& r2, const optional<Tensor>& gate, const optional<Tensor>& sig_bias,
-                      bool sigmoid, double out_scale) {
+                      bool sigmoid, double out_scale, const optional<Tensor>& part) {
   const int dt = act_dt(q, "q");
   same_dt(out, dt, "out");
   check_cache(k_cache, v_cache, dt, G, DK, DV);
@@ -200,12 +200,19 @@ void window_attention(const Tensor& q, const Tensor& k_cache, const Tensor& v_ca
     ldg = row_stride(*gate, "gate");
     TORCH_CHECK(gate->size(0) == T && gate->size(1) == H * DV, "window_attention: gate shape");
   }
+  float* partp = nullptr;
+  if (part) {  // scratch of the key-split decode form of the sigmoid mode
+    TORCH_CHECK(sigmoid && part->is_cuda() && part->scalar_type() == at::kFloat && part->is_contiguous() &&
+                    part->numel() >= (int64_t)gai_sigmoid_attention_splits(T, S, H) * T * H * DV,
+                "window_attention: split scratch too small");
+    partp = part->data_ptr<float>();
+  }
   gai_window_attention(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), i32(block_tables, "block_tables"),
                        block_tables.size(1), i32(cu_q, "cu_q"), i32(ctx, "ctx"), S, out.data_ptr(), ldo, T, H, G, DK, DV,
                        (float)scale, (float)softcap, (int)window, r1 ? f32(*r1, "r1") : nullptr,
                        r2 ? f32(*r2, "r2") : nullptr, gate ? gate->data_ptr() : nullptr, ldg,
                        sig_bias ? f32(*sig_bias, "sig_bias") : nullptr, sigmoid ? 1 : 0, (float)out_scale, dt,
-                       cur_stream());
+                       cur_stream(), partp);
 }
 
 void token_shift_mix(const Tensor& h, const Tensor& mu, const Tensor& shift_state, const Tensor& cu, const Tensor& slots,
@@ -369,6 +376,7 @@ void gai_bind_seq_ops(pybind11::module_& m) {
   m.def("embed_scale_f32", &embed_scale_f32);
   m.def("qknorm_kv_write", &qknorm_kv_write);
   m.def("window_attention", &window_attention);
+  m.def("sigmoid_attention_splits", [](int64_t T, int64_t S, int64_t H) { return (int64_t)gai_sigmoid_attention_splits(T, S, H); });
   m.def("token_shift_mix", &token_shift_mix);
   m.def("state_tail_write", &state_tail_write);
   m.def("conv_silu", &conv_silu);

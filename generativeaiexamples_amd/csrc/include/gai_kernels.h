@@ -232,7 +232,10 @@ void gai_headnorm_kv_write(const void* q, int ldq, const void* k, int ldk, const
 void gai_window_attention(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int maxb,
                           const int* cu_q, const int* ctx, int S, void* out, int ldo, int T, int H, int G, int DK, int DV,
                           float scale, float softcap, int window, const float* r1, const float* r2, const void* gate,
-                          int ldg, const float* sig_bias, int sig, float out_scale, int dt, hipStream_t st);
+                          int ldg, const float* sig_bias, int sig, float out_scale, int dt, hipStream_t st,
+                          float* part = nullptr);
+// sigmoid-mode decode steps: number of key splits (1: none); part must hold splits * T * H * DV floats
+int gai_sigmoid_attention_splits(int T, int S, int H);
 // recurrent.hip
 void gai_token_shift_mix(const void* h, const float* mu, int NM, const float* shift_state, const int* cu,
                          const int* slots, int S, void* out, int T, int D, int dt, hipStream_t st);

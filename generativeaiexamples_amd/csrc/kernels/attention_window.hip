@@ -177,7 +177,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
     const int* __restrict__ block_tables, int maxb, const int* __restrict__ cu_q, const int* __restrict__ ctx, int S,
     TA* __restrict__ out, int ldo, int TH, int H, int G, int DK, int DV, float scale, float softcap, int window,
     const float* __restrict__ r1, const float* __restrict__ r2, const TA* __restrict__ gate, int ldg, int skip_len,
-    const float* __restrict__ sig_bias, float out_scale) {
+    const float* __restrict__ sig_bias, float out_scale, int nsplit, float* __restrict__ part) {
   extern __shared__ float lds[];
   const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int th = blockIdx.x * 4 + wid;
@@ -204,7 +204,15 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
   float m = -INFINITY, l = 0.f, acc[kMaxVChunks];
 #pragma unroll
   for (int n = 0; n < kMaxVChunks; ++n) acc[n] = 0.f;
-  for (int kb = first & ~15; kb <= pos; kb += 64) {
+  // sigmoid mode, decode steps: the key blocks of a row are dealt out to nsplit waves (blockIdx.y) whose unnormalised
+  // partial sums are added up by sigmoid_split_reduce_kernel - there is no softmax state to merge
+  int kb0 = first & ~15, kb1 = pos;
+  if (SIG && nsplit > 1) {
+    const int nblk = (pos - kb0) / 64 + 1, per = (nblk + nsplit - 1) / nsplit;
+    kb0 += (int)blockIdx.y * per * 64;
+    kb1 = min(pos, kb0 + per * 64 - 1);
+  }
+  for (int kb = kb0; kb <= kb1; kb += 64) {
     const int p = kb + lane;
     const bool valid = p >= first && p <= pos;
     float sc = -INFINITY;
@@ -241,6 +249,15 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
       }
     }
   }
+  if (SIG && nsplit > 1) {
+    float* po = part + ((size_t)blockIdx.y * TH + th) * DV;
+#pragma unroll
+    for (int n = 0; n < kMaxVChunks; ++n) {
+      const int c = lane + 64 * n;
+      if (c < DV) po[c] = acc[n];
+    }
+    return;
+  }
   const float inv_l = SIG ? out_scale : 1.0f / l;
   TA* o = out + (size_t)t * ldo + (size_t)h * DV;
 #pragma unroll
@@ -252,6 +269,18 @@ __global__ __launch_bounds__(256) void window_attention_kernel(
       o[c] = (TA)y;
     }
   }
+}
+
+template <typename TA>
+__global__ __launch_bounds__(256) void sigmoid_split_reduce_kernel(const float* __restrict__ part, int nsplit,
+                                                                   TA* __restrict__ out, int ldo, int T, int HDV,
+                                                                   float out_scale) {
+  const long e = (long)blockIdx.x * 256 + threadIdx.x;
+  if (e >= (long)T * HDV) return;
+  const int t = (int)(e / HDV), c = (int)(e % HDV);
+  float a = 0.f;
+  for (int sp = 0; sp < nsplit; ++sp) a += part[(size_t)sp * T * HDV + e];
+  out[(size_t)t * ldo + c] = (TA)(a * out_scale);
 }
 
 // ---- prompt portions in bf16: query tiles on the matrix cores ------------------------------------------------------
@@ -458,10 +487,18 @@ void gai_headnorm_kv_write(const void* q, int ldq, const void* k, int ldk, const
   GAI_LAUNCH_CHECK();
 }
 
+// Key splits of a sigmoid-mode decode step (every row a single token): enough waves to give each SIMD a few
+int gai_sigmoid_attention_splits(int T, int S, int H) {
+  if (T != S || T * H >= 2048) return 1;
+  int n = 4096 / (T * H);
+  return n > 16 ? 16 : (n < 1 ? 1 : n);
+}
+
 void gai_window_attention(const void* q, const void* k_cache, const void* v_cache, const int* block_tables, int maxb,
                           const int* cu_q, const int* ctx, int S, void* out, int ldo, int T, int H, int G, int DK, int DV,
                           float scale, float softcap, int window, const float* r1, const float* r2, const void* gate,
-                          int ldg, const float* sig_bias, int sig, float out_scale, int dt, hipStream_t st) {
+                          int ldg, const float* sig_bias, int sig, float out_scale, int dt, hipStream_t st,
+                          float* part) {
   if (T == 0 || S == 0) return;
   if (DV > 64 * kMaxVChunks) gai_launch_error(__FILE__, __LINE__, "window_attention: value head size above 256");
   if (H % G) gai_launch_error(__FILE__, __LINE__, "window_attention: heads must be a multiple of kv heads");
@@ -481,16 +518,25 @@ void gai_window_attention(const void* q, const void* k_cache, const void* v_cach
 #undef GAI_WIN
     GAI_LAUNCH_CHECK();
   }
+  const int nsplit = (sig && part) ? gai_sigmoid_attention_splits(T, S, H) : 1;
 #define GAI_ROW(TA, SIG_)                                                                                            \
-  window_attention_kernel<TA, SIG_><<<grid, 256, lds, st>>>((const TA*)q, (const TA*)k_cache, (const TA*)v_cache,    \
-                                                            block_tables, maxb, cu_q, ctx, S, (TA*)out, ldo, TH, H, G, \
-                                                            DK, DV, scale, softcap, window, r1, r2, (const TA*)gate,  \
-                                                            ldg, skip_len, sig_bias, out_scale)
+  window_attention_kernel<TA, SIG_><<<dim3(grid, nsplit), 256, lds, st>>>(                                           \
+      (const TA*)q, (const TA*)k_cache, (const TA*)v_cache, block_tables, maxb, cu_q, ctx, S, (TA*)out, ldo, TH, H, G, \
+      DK, DV, scale, softcap, window, r1, r2, (const TA*)gate, ldg, skip_len, sig_bias, out_scale, nsplit, part)
   if (dt) {
     if (sig) GAI_ROW(float, true); else GAI_ROW(float, false);
   } else {
     if (sig) GAI_ROW(bf16, true); else GAI_ROW(bf16, false);
   }
 #undef GAI_ROW
+  if (nsplit > 1) {
+    const long n = (long)T * H * DV;
+    if (dt)
+      sigmoid_split_reduce_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(part, nsplit, (float*)out, ldo, T,
+                                                                                       H * DV, out_scale);
+    else
+      sigmoid_split_reduce_kernel<bf16><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(part, nsplit, (bf16*)out, ldo, T,
+                                                                                      H * DV, out_scale);
+  }
   GAI_LAUNCH_CHECK();
 }

@@ -93,7 +93,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const TA* __restrict__ x
   }
   const int rel = t - cu[lo];
   const float* st = state + (size_t)slots[lo] * (K - 1) * C;
-  for (int c = threadIdx.x; c < C; c += 256) {
+  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += 256 * gridDim.y) {  // few rows: channel tiles across blockIdx.y
     float a = 0.f;
     for (int i = 0; i < K; ++i) {
       const int src = rel - (K - 1) + i;
@@ -1007,10 +1007,11 @@ void gai_state_tail_write(const void* x, int ldx, float* state, const int* cu, c
 void gai_conv_silu(const void* x, int ldx, const float* w, const float* state, const int* cu, const int* slots, int S,
                    float* y, int T, int C, int K, int dt, hipStream_t st, const float* bias, int act) {
   if (T == 0) return;
+  const dim3 grid(T, T <= 256 ? (unsigned)((C + 255) / 256 < 16 ? (C + 255) / 256 : 16) : 1u);
   if (dt)
-    conv_silu_kernel<float><<<T, 256, 0, st>>>((const float*)x, ldx, w, state, cu, slots, S, y, C, K, bias, act);
+    conv_silu_kernel<float><<<grid, 256, 0, st>>>((const float*)x, ldx, w, state, cu, slots, S, y, C, K, bias, act);
   else
-    conv_silu_kernel<bf16><<<T, 256, 0, st>>>((const bf16*)x, ldx, w, state, cu, slots, S, y, C, K, bias, act);
+    conv_silu_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, ldx, w, state, cu, slots, S, y, C, K, bias, act);
   GAI_LAUNCH_CHECK();
 }
 

@@ -1147,7 +1147,7 @@ def window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H: int, G: in
                                     r1, r2, gate)
     out = torch.empty(q.shape[0], H * DV, dtype=q.dtype, device=q.device)
     native().window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, out, H, G, DK, DV, float(scale),
-                              float(softcap or 0.0), int(window or 0), r1, r2, gate, None, False, 1.0)
+                              float(softcap or 0.0), int(window or 0), r1, r2, gate, None, False, 1.0, None)
     return out
 
 
@@ -1163,8 +1163,12 @@ def sigmoid_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, H: int, G: i
         return _into(out, y)
     if out is None:
         out = torch.empty(q.shape[0], H * DV, dtype=q.dtype, device=q.device)
+    # decode steps of few rows: the keys of a row are split over several waves, partial sums in a scratch
+    T, S = q.shape[0], ctx.numel()
+    ns = native().sigmoid_attention_splits(T, S, H)
+    part = torch.empty(ns * T * H * DV, dtype=torch.float32, device=q.device) if ns > 1 else None
     native().window_attention(q, k_cache, v_cache, block_tables, cu_q, ctx, out, H, G, DK, DV, float(scale), 0.0,
-                              int(window or 0), None, None, None, bias, True, float(out_scale))
+                              int(window or 0), None, None, None, bias, True, float(out_scale), part)
     return out
 
 
