@@ -520,7 +520,7 @@ __global__ __launch_bounds__(256) void rglru_gates_kernel(const float* __restric
 #pragma unroll
     for (int tt = 0; tt < kGT; ++tt) ar[tt] = ai[tt] = 0.f;
     int k = 0;
-    if ((BS & 3) == 0) {  // four input channels a round: one 16-byte LDS broadcast per token instead of four reads
+    if ((BS & 3) == 0) {  // four input channels per iteration: one 16-byte LDS broadcast per token instead of four reads
       for (; k < BS; k += 4) {
         float xa[4], xi[4];
 #pragma unroll
