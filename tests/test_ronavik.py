@@ -162,11 +162,10 @@ def test_ops_against_oracle_mechanisms(device, dtype):
     W, nb, T = 30, 3, 9
     u, ya = rn(T, W), rn(T, W)
     wa, wi, ba, bi, lam = rn(nb, 10, 10), rn(nb, 10, 10), rn(W), rn(W), rn(W) - 2
-    a, b = ops.rglru_gates(u.to(dev), wa.transpose(1, 2).contiguous().to(dev), ba.to(dev), wi.transpose(1, 2).contiguous().to(dev),
-                           bi.to(dev), lam.to(dev), 8.0)
-    r_ = torch.cat([torch.sigmoid(u[:, 10 * i:10 * i + 10].double() @ wa[i].double().T) for i in range(nb)], 1)
-    r_ = torch.sigmoid(torch.cat([u[:, 10 * i:10 * i + 10].double() @ wa[i].double().T for i in range(nb)], 1) + ba.double())
-    i_ = torch.sigmoid(torch.cat([u[:, 10 * i:10 * i + 10].double() @ wi[i].double().T for i in range(nb)], 1) + bi.double())
+    wa_t, wi_t = wa.transpose(1, 2).contiguous().to(dev), wi.transpose(1, 2).contiguous().to(dev)
+    a, b = ops.rglru_gates(u.to(dev), wa_t, ba.to(dev), wi_t, bi.to(dev), lam.to(dev), 8.0)
+    blocks = lambda w: torch.cat([u[:, 10 * i:10 * i + 10].double() @ w[i].double().T for i in range(nb)], 1)  # noqa: E731
+    r_, i_ = torch.sigmoid(blocks(wa) + ba.double()), torch.sigmoid(blocks(wi) + bi.double())
     a_ = torch.exp(-8.0 * r_ * torch.nn.functional.softplus(lam.double()))
     assert torch.allclose(a.cpu().double(), a_, atol=1e-5)
     assert torch.allclose(b.cpu().double(), torch.sqrt(1 - a_ ** 2) * i_ * u.double(), atol=1e-5)
